@@ -26,7 +26,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import KVNeed, PagedNeed, StateNeed
+from ..parts.base import KVNeed, PagedNeed, StateNeed, CompoundNeed
 from .pages import PagePool, CacheFull
 
 
@@ -66,23 +66,21 @@ class CacheManager:
                  max_step_tokens=None, allocate=True):
         self.page_size, self.max_requests, self.dtype, self.device = page_size, max_requests, dtype, torch.device(device)
         self.kv_groups, self.state_groups = [], []     # dicts: need, entries, pool / need, entries
-        self.binding = []                              # per schedule entry: None | (kind, group, index, writes)
+        # per schedule entry: None | (kind, group, index, writes) | a list of those (an entry with a CompoundNeed)
+        self.binding = []
         for position, need in enumerate(needs):
             if need is None:
                 self.binding.append(None)
             elif isinstance(need, tuple) and need[0] == 'shared':
-                kind, group, index, _ = self.binding[need[1]]
-                self.binding.append((kind, group, index, False))
-            elif isinstance(need, (KVNeed, PagedNeed)):
-                group = self._group(self.kv_groups, need)
-                self.binding.append(('kv', group, len(self.kv_groups[group]['entries']), True))
-                self.kv_groups[group]['entries'].append(position)
-            elif isinstance(need, StateNeed):
-                group = self._group(self.state_groups, need)
-                self.binding.append(('state', group, len(self.state_groups[group]['entries']), True))
-                self.state_groups[group]['entries'].append(position)
+                owner = self.binding[need[1]]
+                if isinstance(owner, list):
+                    self.binding.append([(kind, group, index, False) for kind, group, index, _ in owner])
+                else:
+                    self.binding.append((owner[0], owner[1], owner[2], False))
+            elif isinstance(need, CompoundNeed):
+                self.binding.append([self._bind(position, one) for one in need.needs])
             else:
-                raise TypeError(f'unknown cache need {need!r}')
+                self.binding.append(self._bind(position, need))
         pages = num_pages if isinstance(num_pages, (list, tuple)) else [num_pages] * len(self.kv_groups)
         if len(pages) != len(self.kv_groups):
             raise ValueError(f'{len(self.kv_groups)} page groups, {len(pages)} page counts')
@@ -93,6 +91,17 @@ class CacheManager:
         self.slots, self.computed, self.limits = {}, {}, {}
         if allocate:
             self._allocate()
+
+    def _bind(self, position, need):
+        if isinstance(need, (KVNeed, PagedNeed)):
+            group = self._group(self.kv_groups, need)
+            self.kv_groups[group]['entries'].append(position)
+            return ('kv', group, len(self.kv_groups[group]['entries']) - 1, True)
+        if isinstance(need, StateNeed):
+            group = self._group(self.state_groups, need)
+            self.state_groups[group]['entries'].append(position)
+            return ('state', group, len(self.state_groups[group]['entries']) - 1, True)
+        raise TypeError(f'unknown cache need {need!r}')
 
     @staticmethod
     def _group(groups, need):
@@ -215,22 +224,18 @@ class CacheManager:
 
     # ------------------------------------------------------------------ views
     def views(self):
-        """One view per schedule entry (None where the mixer keeps nothing)."""
-        out = []
-        for bound in self.binding:
-            if bound is None:
-                out.append(None)
-                continue
+        """One view per schedule entry (None where the entry keeps nothing; a tuple of views for an entry with a
+        ``CompoundNeed``, in the order of its needs)."""
+        def view(bound):
             kind, group, index, writes = bound
             if kind == 'kv':
                 g = self.kv_groups[group]
                 if isinstance(g['need'], PagedNeed):
-                    out.append(PagedView({name: t[index] for name, t in g['tensors'].items()}, self.page_size, writes, group))
-                else:
-                    out.append(KVView(g['k'][index], g['v'][index], self.page_size, writes, group))
-            else:
-                out.append(StateView(self.state_groups[group]['state'][index], writes, group))
-        return out
+                    return PagedView({name: t[index] for name, t in g['tensors'].items()}, self.page_size, writes, group)
+                return KVView(g['k'][index], g['v'][index], self.page_size, writes, group)
+            return StateView(self.state_groups[group]['state'][index], writes, group)
+        return [None if bound is None else tuple(view(one) for one in bound) if isinstance(bound, list) else view(bound)
+                for bound in self.binding]
 
     def bytes_per_token(self):
         size = torch.empty((), dtype=self.dtype).element_size()

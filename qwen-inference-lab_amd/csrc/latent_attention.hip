@@ -9,6 +9,10 @@
 // Every head reads the same cached row: one staged tile of keys serves all heads of a block.
 // The sink: a logit s_h with no key and no value; it enters the running maximum and the denominator once
 // (running state starts at maximum s_h, sum 1, result 0).
+// A window w > 0: the row at position p sees the keys j with 0 <= p - j < w only (w <= 0: every key j <= p).
+// An output gate: head h's result of row n is multiplied by gate[n, h] (a float32 factor per row and head, made by
+// the prepare kernel as the sigmoid of `gates` more columns of the stacked down product); a factor per head commutes
+// with W_uv,h, so it is applied here, to the weighted sum of latents.
 #include "common.h"
 #include "partials.h"
 
@@ -16,16 +20,18 @@
 // Step 1 of the mixer, after the stacked down products x = [W_dq h ; W_dkv h] (q_rank + rank + rot columns):
 //   cq = x[:q_rank] / sqrt(mean(.^2) + eps) * wq                     -> cq_out (T)
 //   c  = x[q_rank : q_rank + rank] / sqrt(mean(.^2) + eps) * wc      -> latent cache at the row's slot
-//   kr = rotate(x[q_rank + rank :], position)                        -> rope cache at the row's slot
+//   kr = rotate(x[q_rank + rank : q_rank + rank + rot], position)    -> rope cache at the row's slot
+//   g  = sigmoid(x[q_rank + rank + rot :])   (`gates` columns, if any)  -> gate_out [n, gates] float32
 // Rotation of a vector of `rot` elements: element i pairs with i + rot / 2, angle position * freq[i].
 template <typename TD, typename T>
 __global__ void latent_prepare_kernel(const TD* __restrict__ x, int splits, size_t split_stride, const float* __restrict__ wq,
                                       const float* __restrict__ wc, const float* __restrict__ freq,
                                       const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ cq_out,
-                                      T* __restrict__ latent, T* __restrict__ rope, int q_rank, int rank, int rot, float eps, int held) {
-  extern __shared__ float sums[];                     // [q_rank + rank + rot] when `held`: the row, its partial sums added
+                                      T* __restrict__ latent, T* __restrict__ rope, float* __restrict__ gate_out, int q_rank,
+                                      int rank, int rot, int gates, float eps, int held) {
+  extern __shared__ float sums[];                     // [q_rank + rank + rot + gates] when `held`: the row, its partial sums added
   __shared__ float scratch[16];
-  const int n = blockIdx.x, total = q_rank + rank + rot;
+  const int n = blockIdx.x, total = q_rank + rank + rot + gates;
   const size_t at = (size_t)n * total;
   if (held) {                                         // every element is read from memory once, all reads side by side
     for (int i = threadIdx.x; i < total; i += blockDim.x) sums[i] = parts_sum(x, at + i, splits, split_stride);
@@ -39,6 +45,8 @@ __global__ void latent_prepare_kernel(const TD* __restrict__ x, int splits, size
   sc = block_sum(sc, scratch);
   const float rq = 1.f / sqrtf(sq / (float)q_rank + eps), rc = 1.f / sqrtf(sc / (float)rank + eps);
   for (int i = threadIdx.x; i < q_rank; i += blockDim.x) st(cq_out + (size_t)n * q_rank + i, value(i) * rq * wq[i]);
+  for (int i = threadIdx.x; i < gates; i += blockDim.x)
+    gate_out[(size_t)n * gates + i] = 1.f / (1.f + expf(-value(q_rank + rank + rot + i)));
   if (!slots) return;
   const size_t slot = (size_t)slots[n];
   for (int i = threadIdx.x; i < rank; i += blockDim.x) st(latent + slot * rank + i, value(q_rank + i) * rc * wc[i]);
@@ -172,8 +180,9 @@ template <typename TC>
 __global__ void __launch_bounds__(LA_THREADS)
 latent_attention_kernel(const float* __restrict__ q, const TC* __restrict__ latent, const TC* __restrict__ rope,
                         const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
-                        const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out,
-                        int heads, int group, int rank, int rot, int page_size, int kt, float scale) {
+                        const int* __restrict__ positions, const float* __restrict__ sink, const float* __restrict__ gate,
+                        float* __restrict__ out, int heads, int group, int rank, int rot, int page_size, int kt, float scale,
+                        int window) {
   extern __shared__ float lds[];
   const int d = rank + rot, pad = d + 1;
   float* qs = lds;                                   // [group][d]
@@ -195,7 +204,8 @@ latent_attention_kernel(const float* __restrict__ q, const TC* __restrict__ late
   for (int a = 0; a < LA_ACC; ++a) acc[a] = 0.f;
   const int owned = live * rank;
 
-  for (int j0 = 0; j0 <= position; j0 += kt) {
+  const int first = window > 0 ? max(0, position - window + 1) : 0;     // the oldest key the row sees
+  for (int j0 = first; j0 <= position; j0 += kt) {
     const int keys = min(kt, position + 1 - j0);
     __syncthreads();                                 // the last tile's reads are done (and qs / top / den are written)
     for (int idx = tid; idx < keys * d; idx += LA_THREADS) {
@@ -251,7 +261,8 @@ latent_attention_kernel(const float* __restrict__ q, const TC* __restrict__ late
     const int e = tid + a * LA_THREADS;
     if (e < owned) {
       const int h = e / rank, c = e - h * rank;
-      out[((size_t)n * heads + h0 + h) * rank + c] = acc[a] / den[h];
+      const float factor = gate ? gate[(size_t)n * heads + h0 + h] : 1.f;
+      out[((size_t)n * heads + h0 + h) * rank + c] = acc[a] / den[h] * factor;
     }
   }
 }
@@ -272,16 +283,18 @@ static void latent_plan(int heads, int rank, int rot, int* group, int* kt, size_
 extern "C" {
 
 int qil_latent_prepare(const void* x, int x_dtype, int splits, const float* wq, const float* wc, const float* freq,
-                       const int* positions, const int* slots, void* cq_out, void* latent, void* rope, int n, int q_rank,
-                       int rank, int rot, float eps, int dtype, hipStream_t s) {
+                       const int* positions, const int* slots, void* cq_out, void* latent, void* rope, float* gate_out,
+                       int n, int q_rank, int rank, int rot, int gates, float eps, int dtype, hipStream_t s) {
   if (n == 0) return 0;
-  if (q_rank < 1 || rank < 1 || rot < 2 || rot % 2 || splits < 1 || (x_dtype == QIL_BF16 && splits != 1)) return -1;
-  const size_t stride = (size_t)n * (q_rank + rank + rot);
-  const size_t row_bytes = (size_t)(q_rank + rank + rot) * sizeof(float);
+  if (q_rank < 1 || rank < 1 || rot < 2 || rot % 2 || splits < 1 || (x_dtype == QIL_BF16 && splits != 1) || gates < 0 ||
+      (gates > 0 && !gate_out))
+    return -1;
+  const size_t stride = (size_t)n * (q_rank + rank + rot + gates);
+  const size_t row_bytes = (size_t)(q_rank + rank + rot + gates) * sizeof(float);
   const int held = row_bytes <= 48 * 1024;            // the row's sums fit in LDS
 #define QIL_LP(TD, T)                                                                                               \
   hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(256), held ? row_bytes : 0, s, (const TD*)x, splits, \
-                     stride, wq, wc, freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, q_rank, rank, rot, eps, held)
+                     stride, wq, wc, freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, gate_out, q_rank, rank, rot, gates, eps, held)
   if (dtype == QIL_F32) {
     if (x_dtype != QIL_F32) return -1;
     QIL_LP(float, float);
@@ -349,8 +362,9 @@ int qil_latent_attention_takes(int heads, int rank, int rot) {
 }
 
 int qil_latent_attention(const float* q, const void* latent, const void* rope, const int* tables, int table_stride,
-                         const int* row_seq, const int* positions, const float* sink, float* out, int n, int heads,
-                         int rank, int rot, int page_size, float scale, int cache_dtype, hipStream_t s) {
+                         const int* row_seq, const int* positions, const float* sink, const float* gate, float* out, int n,
+                         int heads, int rank, int rot, int page_size, float scale, int window, int cache_dtype,
+                         hipStream_t s) {
   if (n == 0) return 0;
   if (!qil_latent_attention_takes(heads, rank, rot) || page_size < 1) return -1;
   int group, kt;
@@ -359,12 +373,12 @@ int qil_latent_attention(const float* q, const void* latent, const void* rope, c
   dim3 grid(n, (heads + group - 1) / group);
   if (cache_dtype == QIL_F32)
     hipLaunchKernelGGL(latent_attention_kernel<float>, grid, dim3(LA_THREADS), lds, s, q, (const float*)latent,
-                       (const float*)rope, tables, table_stride, row_seq, positions, sink, out, heads, group, rank, rot,
-                       page_size, kt, scale);
+                       (const float*)rope, tables, table_stride, row_seq, positions, sink, gate, out, heads, group, rank,
+                       rot, page_size, kt, scale, window);
   else
     hipLaunchKernelGGL(latent_attention_kernel<bf16_t>, grid, dim3(LA_THREADS), lds, s, q, (const bf16_t*)latent,
-                       (const bf16_t*)rope, tables, table_stride, row_seq, positions, sink, out, heads, group, rank, rot,
-                       page_size, kt, scale);
+                       (const bf16_t*)rope, tables, table_stride, row_seq, positions, sink, gate, out, heads, group, rank,
+                       rot, page_size, kt, scale, window);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

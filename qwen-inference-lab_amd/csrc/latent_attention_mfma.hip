@@ -15,6 +15,9 @@
 //
 // With few blocks the keys go in parts (grid.z): a block leaves (reference, sum, unnormalised result) per column and
 // part, and latent_merge_kernel finishes, which is also where the sink enters then.
+// A window w > 0 hides the keys j <= position - w of a row: a block begins at the oldest key its first row sees, a
+// part that no row of the block sees is left out, and the merge reads the parts between a row's oldest key and its
+// position.  An output gate (a float32 factor per row and head) multiplies the finished column.
 //
 // Takes rank % 16 == 0, rot % 8 == 0, rank + rot <= 640, rank <= 512; other sizes run on the general kernel.
 #include "common.h"
@@ -38,9 +41,9 @@ __global__ void __launch_bounds__(LM_THREADS, SPLIT ? 2 : 1)
 latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ latent, const bf16_t* __restrict__ rope,
                    const int* __restrict__ tables, int table_stride, const int* __restrict__ cu_seqlens,
                    const int* __restrict__ seq_starts, int n_seqs, int single, const float* __restrict__ sink,
-                   float* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_m,
+                   const float* __restrict__ gate, float* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_m,
                    float* __restrict__ part_l, int heads, int rank, int rot, int page_size, float scale, int rt, int hb,
-                   int P, int parts) {
+                   int P, int parts, int window) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int d = rank + rot;
   const int qf = EXACT ? QF : (d + 31) / 32, vt = EXACT ? VT : rank / 16;
@@ -66,7 +69,8 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   const int last_pos = start + r0 + rows_here - 1;
   const int h0 = blockIdx.y * hb, heads_here = min(hb, heads - h0);
   const int part = blockIdx.z;
-  const int begin = part * P, end = min((part + 1) * P, last_pos + 1);
+  const int oldest = window > 0 ? max(0, start + r0 - window + 1) : 0;     // of the tile's first row, which sees furthest back
+  const int begin = max(part * P, oldest), end = min((part + 1) * P, last_pos + 1);
   if (begin >= end) return;                                 // no row of the tile sees this part; the merge does not read it
   const int* table = tables + (size_t)s * table_stride;
 
@@ -79,6 +83,7 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   const int t0 = SPLIT ? wave * VTW : 0;
   const int grow = seq_row0 + r0 + (valid ? ci : 0), head = h0 + (valid ? ch : 0);
   const int pos = valid ? start + r0 + ci : -1;
+  const int low = window > 0 ? pos - window + 1 : 0;        // the column's oldest visible key (<= 0: from the start)
   const size_t gcol = (size_t)grow * heads + head;
 
   bf16x8 qb[QF];
@@ -198,7 +203,7 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = j0 + 8 * kb + 4 * jt + i;
-        const float v = (key <= pos && key < end) ? sc[jt][i] * scale : -INFINITY;
+        const float v = (key <= pos && key >= low && key < end) ? sc[jt][i] * scale : -INFINITY;
         sc[jt][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -254,7 +259,7 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   l += __shfl_xor(l, 32, QIL_WAVE);
   if (!valid) return;
   if (parts == 1) {
-    const float inv = 1.f / l;
+    const float inv = (gate ? gate[gcol] : 1.f) / l;
     float* dst = out + gcol * rank + 16 * t0 + 4 * kb;
 #pragma unroll
     for (int t = 0; t < VTW; ++t)
@@ -279,34 +284,35 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
 // for no value that another read has to bring first.
 __global__ void latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
                                     const float* __restrict__ part_l, const int* __restrict__ positions,
-                                    const float* __restrict__ sink, float* __restrict__ out, int heads, int rank, int P,
-                                    int parts) {
+                                    const float* __restrict__ sink, const float* __restrict__ gate,
+                                    float* __restrict__ out, int heads, int rank, int P, int parts, int window) {
   extern __shared__ float weight[];
   __shared__ float scratch[16];
   const int n = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
   const size_t column = (size_t)n * heads + h;
   const int reached = min(parts, positions[n] / P + 1);
+  const int from = window > 0 ? max(0, positions[n] - window + 1) / P : 0;     // the part of the row's oldest visible key
   const float floor_ = sink ? sink[h] : -INFINITY;
   float top = floor_;
-  for (int p = tid; p < reached; p += nt) {
+  for (int p = from + tid; p < reached; p += nt) {
     const float mp = part_m[column * parts + p];
     weight[p] = mp;
     top = fmaxf(top, mp);
   }
   top = block_max(top, scratch);
   float below = (sink && tid == 0) ? expf(floor_ - top) : 0.f;
-  for (int p = tid; p < reached; p += nt) {                 // a thread rereads only what it wrote
+  for (int p = from + tid; p < reached; p += nt) {          // a thread rereads only what it wrote
     const float mp = weight[p], w = mp > -INFINITY ? expf(mp - top) : 0.f;
     weight[p] = w;
     below += w * part_l[column * parts + p];
   }
   below = block_sum(below, scratch);                        // its barriers also publish the weights
-  const float inv = 1.f / below;
+  const float inv = (gate ? gate[column] : 1.f) / below;
   const float* acc_p = part_acc + column * parts * rank;
   for (int c = tid; c < rank; c += nt) {
     float acc = 0.f;
 #pragma unroll 4
-    for (int p = 0; p < reached; ++p) acc += weight[p] * acc_p[(size_t)p * rank + c];
+    for (int p = from; p < reached; ++p) acc += weight[p] * acc_p[(size_t)p * rank + c];
     out[column * rank + c] = acc * inv;
   }
 }
@@ -319,8 +325,9 @@ static int lm_lds_bytes(int rank, int rot) {
 template <int QF, int VT, bool EXACT, bool SPLIT>
 static int lm_launch(dim3 grid, size_t lds, hipStream_t s, const float* q, const bf16_t* latent, const bf16_t* rope,
                      const int* tables, int table_stride, const int* cu_seqlens, const int* seq_starts, int n_seqs,
-                     int single, const float* sink, float* out, float* part_acc, float* part_m, float* part_l, int heads,
-                     int rank, int rot, int page_size, float scale, int rt, int hb, int P, int parts) {
+                     int single, const float* sink, const float* gate, float* out, float* part_acc, float* part_m,
+                     float* part_l, int heads, int rank, int rot, int page_size, float scale, int rt, int hb, int P, int parts,
+                     int window) {
   auto kernel = latent_mfma_kernel<QF, VT, EXACT, SPLIT>;
   static bool raised = false;                                // per instantiation
   if (lds > 64 * 1024 && !raised) {
@@ -329,8 +336,8 @@ static int lm_launch(dim3 grid, size_t lds, hipStream_t s, const float* q, const
     raised = true;
   }
   hipLaunchKernelGGL(kernel, grid, dim3(LM_THREADS), lds, s, q, latent, rope, tables, table_stride, cu_seqlens, seq_starts,
-                     n_seqs, single, sink, out, part_acc, part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P,
-                     parts);
+                     n_seqs, single, sink, gate, out, part_acc, part_m, part_l, heads, rank, rot, page_size, scale, rt, hb,
+                     P, parts, window);
   return 0;
 }
 
@@ -343,8 +350,10 @@ int qil_latent_mfma_takes(int heads, int rank, int rot) {
 
 // (rows a block, heads a block, keys a part, parts) for a step: blocks of up to 64 columns (16 where every sequence
 // has one row: the split form); the keys in parts of at least 64 while the blocks are fewer than two a compute unit.
-void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max_context, int* rt, int* hb, int* P,
-                          int* parts) {
+// With a window a block walks at most the window and its own rows, so that span is what the parts divide; parts
+// still count from key 0 (those outside every row's window do nothing).
+void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max_context, int window, int* rt, int* hb,
+                          int* P, int* parts) {
   const int most = single ? 16 : 64;                          // single rows: one wave's columns a block
   *hb = heads < most ? heads : most;
   *rt = single ? 1 : (64 / *hb > 0 ? 64 / *hb : 1);
@@ -352,7 +361,9 @@ void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max
   const long blocks = (long)tiles * ((heads + *hb - 1) / *hb);
   int want = (int)((2 * QIL_CUS + blocks - 1) / blocks);
   if (want < 1) want = 1;
-  int part = ((max_context + want - 1) / want + 31) / 32 * 32;
+  int span = max_context;
+  if (window > 0 && window + *rt - 1 < span) span = window + *rt - 1;
+  int part = ((span + want - 1) / want + 31) / 32 * 32;
   if (part < 64) part = 64;                                   // two steps a block: shorter parts cost more in the merge than they save
   *P = part;
   *parts = (max_context + part - 1) / part;
@@ -366,9 +377,9 @@ size_t qil_latent_mfma_workspace(int n_rows, int heads, int rank, int parts) {
 // q float32 [n_rows, heads, rank + rot]; out float32 [n_rows, heads, rank]; workspace as qil_latent_mfma_workspace says.
 // single: every sequence has one row (n_seqs == n_rows).  rt, hb, P, parts: as qil_latent_mfma_plan gave them.
 int qil_latent_mfma(const float* q, const void* latent, const void* rope, const int* tables, int table_stride,
-                    const int* cu_seqlens, const int* seq_starts, const int* positions, const float* sink, float* out,
-                    float* workspace, int n_rows, int n_seqs, int single, int heads, int rank, int rot, int page_size,
-                    float scale, int rt, int hb, int P, int parts, hipStream_t s) {
+                    const int* cu_seqlens, const int* seq_starts, const int* positions, const float* sink,
+                    const float* gate, float* out, float* workspace, int n_rows, int n_seqs, int single, int heads, int rank,
+                    int rot, int page_size, float scale, int window, int rt, int hb, int P, int parts, hipStream_t s) {
   if (n_rows == 0) return 0;
   if (!qil_latent_mfma_takes(heads, rank, rot) || page_size < 1 || rt < 1 || hb < 1 || rt * hb > (single ? 16 : 64) || P < 32 || P % 32 ||
       parts < 1 || parts > 8192 || (single && n_seqs != n_rows) || (parts > 1 && !workspace))
@@ -383,7 +394,8 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
   int status;
 #define QIL_LM_ARGS                                                                                                  \
   grid, lds, s, q, (const bf16_t*)latent, (const bf16_t*)rope, tables, table_stride, cu_seqlens, seq_starts, n_seqs, \
-      single, parts == 1 ? sink : nullptr, out, part_acc, part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P, parts
+      single, parts == 1 ? sink : nullptr, parts == 1 ? gate : nullptr, out, part_acc, part_m, part_l, heads, rank, rot,     \
+      page_size, scale, rt, hb, P, parts, window
 #define QIL_LM(QF, VT, EXACT) \
   status = single ? lm_launch<QF, VT, EXACT, true>(QIL_LM_ARGS) : lm_launch<QF, VT, EXACT, false>(QIL_LM_ARGS)
   if (qf == 18 && vt == 32) QIL_LM(18, 32, true);
@@ -395,7 +407,7 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
   if (status) return status;
   if (parts > 1)
     hipLaunchKernelGGL(latent_merge_kernel, dim3(n_rows, heads), dim3(rank >= 256 ? 256 : 64), parts * sizeof(float), s, part_acc, part_m,
-                       part_l, positions, sink, out, heads, rank, P, parts);
+                       part_l, positions, sink, gate, out, heads, rank, P, parts, window);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

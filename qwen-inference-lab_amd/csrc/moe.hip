@@ -1,8 +1,9 @@
 // A routed feed-forward (mixture of experts): the router, the grouping of (token, chosen expert) pairs by expert, the
 // experts' two products on the matrix cores, and the weighted sum.
 //
-//   route    (two kernels: the logits, then the choice) per token: logits z = W_r h in float32 (W_r float32, h as it comes), scores s = softmax(z) over all
-//            outputs; choice scores c = s + correction; the outputs form `groups` equal groups of neighbours, a
+//   route    (two kernels: the logits, then the choice) per token: logits z = W_r h (+ a stored bias) in float32 (W_r float32, h as it comes), scores s = softmax(z) over all
+//            outputs; choice scores c = s + correction (without a correction the choice goes by the logits themselves,
+//            which order the outputs as their scores do and do not underflow); the outputs form `groups` equal groups of neighbours, a
 //            group's score is its largest c, and only the `keep` best groups stay (the others' c count as -inf);
 //            the `top` largest c are chosen (lowest index first among equals); the weights are their s, optionally
 //            divided by their sum.  The last `identity` outputs are experts without tensors that pass their input.
@@ -83,7 +84,8 @@ moe_logits_kernel(const T* __restrict__ x, int n, int width, const float* __rest
 // The choice from the logits: a wave a row, four rows a block (every wave walks the same steps, so the barriers
 // between a wave's writes to its part of LDS and its reads are met by all).
 __global__ void __launch_bounds__(MOE_ROUTE_THREADS)
-moe_select_kernel(const float* __restrict__ logits, int n, const float* __restrict__ correction, int outputs, int groups,
+moe_select_kernel(const float* __restrict__ logits, int n, const float* __restrict__ bias,
+                  const float* __restrict__ correction, int outputs, int groups,
                   int keep, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weights) {
   extern __shared__ float lds[];                        // per wave: [outputs] scores, [outputs] choice scores, [groups]
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
@@ -93,16 +95,17 @@ moe_select_kernel(const float* __restrict__ logits, int n, const float* __restri
   const int n_row = blockIdx.x * (MOE_ROUTE_THREADS / QIL_WAVE) + wave;
   const bool live = n_row < n;
   const float* z = logits + (size_t)min(n_row, n - 1) * outputs;
+  auto logit = [&](int e) { return z[e] + (bias ? bias[e] : 0.f); };
   float top_logit = -INFINITY;
-  for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, z[e]);
+  for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, logit(e));
   top_logit = wave_max(top_logit);
   float total = 0.f;
-  for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(z[e] - top_logit);
+  for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(logit(e) - top_logit);
   total = wave_sum(total);
   for (int e = lane; e < outputs; e += QIL_WAVE) {
-    const float s = expf(z[e] - top_logit) / total;
+    const float s = expf(logit(e) - top_logit) / total;
     score[e] = s;
-    choice[e] = s + (correction ? correction[e] : 0.f);
+    choice[e] = correction ? s + correction[e] : logit(e);
   }
   __syncthreads();
   if (groups > 1 && keep < groups) {
@@ -498,9 +501,10 @@ int qil_moe_takes(int width, int outputs, int experts, int groups, int keep, int
          (size_t)(MOE_ROUTE_THREADS / QIL_WAVE) * (2 * outputs + groups) * sizeof(float) <= 64 * 1024;
 }
 
-// x [n, width] (dtype), w_router float32 [outputs, width], correction float32 [outputs] or null -> chosen int32
-// [n, top], weights float32 [n, top].  logits: float32 scratch [n, outputs].
-int qil_moe_route(const void* x, int dtype, const float* w_router, const float* correction, float* logits, int* chosen,
+// x [n, width] (dtype), w_router float32 [outputs, width], bias and correction float32 [outputs] or null -> chosen
+// int32 [n, top], weights float32 [n, top].  logits: float32 scratch [n, outputs].
+int qil_moe_route(const void* x, int dtype, const float* w_router, const float* bias, const float* correction,
+                  float* logits, int* chosen,
                   float* weights, int n, int width, int outputs, int groups, int keep, int top, int renormalize,
                   hipStream_t s) {
   if (n == 0) return 0;
@@ -516,7 +520,7 @@ int qil_moe_route(const void* x, int dtype, const float* w_router, const float* 
   const int per_block = MOE_ROUTE_THREADS / QIL_WAVE;
   const size_t lds = (size_t)per_block * (2 * outputs + groups) * sizeof(float);
   hipLaunchKernelGGL(moe_select_kernel, dim3((n + per_block - 1) / per_block), dim3(MOE_ROUTE_THREADS), lds, s, logits, n,
-                     correction, outputs, groups, keep, top, renormalize, chosen, weights);
+                     bias, correction, outputs, groups, keep, top, renormalize, chosen, weights);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -1,0 +1,88 @@
+// A sub-layer's output that joins the float32 residual stream as its norm, scaled per channel, and optionally a
+// weighted average over the results of all layers so far:
+//
+//   z      = norm(y) * w + b                 norm: (y - mean) / sqrt(mean((y - mean)^2) + eps) (CENTRE), or
+//                                            y / sqrt(mean(y^2) + eps); w, b, the channel scale ls: float32 or absent
+//   X      = stream + ls * z                 the layer's result so far
+//   depth > 0:  history[depth - 1] = X;  stream = sum_(j < depth) mix[j] * history[j]   (the new X is the last term)
+//   else:       stream = X
+//   out    = stream rounded to T             (if asked for: what the next sub-layer's products read)
+//
+// y: one array of the model's type or float32 partial sums [splits][rows][width]; everything else is float32.
+// One block per row; the row of y is held in LDS between the passes (statistics in two passes: the variance is that
+// of the deviations).
+#include "common.h"
+#include "partials.h"
+
+template <typename TD, typename T, int CENTRE>
+__global__ void post_norm_scale_add_kernel(float* __restrict__ stream, const TD* __restrict__ y, int splits, size_t split_stride,
+                                           const float* __restrict__ weight, const float* __restrict__ bias,
+                                           const float* __restrict__ channel_scale, float eps, T* __restrict__ out,
+                                           float* __restrict__ history, size_t history_stride, int depth,
+                                           const float* __restrict__ mix, int width) {
+  extern __shared__ float row[];                      // [width]
+  __shared__ float scratch[16];
+  const size_t at = (size_t)blockIdx.x * width;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = parts_sum(y, at + i, splits, split_stride);
+    row[i] = v;                                       // a thread rereads only what it wrote
+    sum += v;
+  }
+  float mean = 0.f;
+  if (CENTRE) mean = block_sum(sum, scratch) / (float)width;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float c = row[i] - mean;
+    squares += c * c;
+  }
+  squares = block_sum(squares, scratch);
+  const float scale = 1.f / sqrtf(squares / (float)width + eps);
+  float* x = stream + at;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float z = (row[i] - mean) * scale;
+    if (weight) z *= weight[i];
+    if (bias) z += bias[i];
+    if (channel_scale) z *= channel_scale[i];
+    float v = x[i] + z;
+    if (depth > 0) {
+      history[(size_t)(depth - 1) * history_stride + at + i] = v;
+      float mixed = 0.f;
+      for (int j = 0; j + 1 < depth; ++j) mixed += mix[j] * history[(size_t)j * history_stride + at + i];
+      v = mixed + mix[depth - 1] * v;
+    }
+    x[i] = v;
+    if (out) st(out + at + i, v);
+  }
+}
+
+extern "C" {
+
+// stream float32 [n, width], changed in place.  y: y_dtype QIL_BF16 (one array, splits == 1) or QIL_F32
+// ([splits][n][width] partial sums).  weight, bias, channel_scale: float32 [width] or null.  out: null, or [n, width] of
+// out_dtype (the new stream, rounded).  history: null (depth 0), or float32 [>= depth][n][width] whose entries
+// 0 .. depth - 2 are read and whose entry depth - 1 is written; mix float32 [depth].
+int qil_post_norm_scale_add(float* stream, const void* y, int y_dtype, int splits, const float* weight, const float* bias,
+                            const float* channel_scale, float eps, int centre, void* out, int out_dtype, float* history,
+                            int depth, const float* mix, int n, int width, hipStream_t s) {
+  if (n == 0) return 0;
+  if (width < 1 || splits < 1 || (y_dtype == QIL_BF16 && splits != 1) || depth < 0 || (depth > 0 && (!history || !mix)) ||
+      (size_t)width * sizeof(float) > 64 * 1024)
+    return -1;
+  const size_t stride = (size_t)n * width, lds = (size_t)width * sizeof(float);
+  const int threads = width >= 2048 ? 512 : width >= 512 ? 256 : width >= 128 ? 128 : 64;
+#define QIL_POST_LAUNCH(TD, T, C)                                                                                      \
+  hipLaunchKernelGGL((post_norm_scale_add_kernel<TD, T, C>), dim3(n), dim3(threads), lds, s, stream, (const TD*)y, splits, \
+                     stride, weight, bias, channel_scale, eps, (T*)out, history, stride, depth, mix, width)
+#define QIL_POST_CASE(TD, T) do { if (centre) QIL_POST_LAUNCH(TD, T, 1); else QIL_POST_LAUNCH(TD, T, 0); } while (0)
+  if (out_dtype == QIL_F32) {
+    if (y_dtype == QIL_F32) QIL_POST_CASE(float, float); else QIL_POST_CASE(bf16_t, float);
+  } else {
+    if (y_dtype == QIL_F32) QIL_POST_CASE(float, bf16_t); else QIL_POST_CASE(bf16_t, bf16_t);
+  }
+#undef QIL_POST_CASE
+#undef QIL_POST_LAUNCH
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -163,7 +163,7 @@ class ModelRunner:
             single_rows=part('single_rows') if max(counts) > 1 else None, max_query=max(counts),
             max_context=max_context or facts['max_context'], host_cu_seqlens=facts['cu'], host_starts=facts['starts'],
             host_slots=facts['slots'], requests=[e.request for e in entries], tile_seqs=facts['tile_seqs'])
-        for view in self.views:
+        for view in (one for view in self.views for one in (view if isinstance(view, tuple) else (view,))):
             if view is not None and hasattr(view, 'block_tables'):
                 view.block_tables = part(f'tables{view.group}').view(s, facts['widths'][view.group])
                 view.slots = part(f'token_slots{view.group}')

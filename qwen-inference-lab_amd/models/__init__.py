@@ -2,3 +2,4 @@
 from . import qwen3  # noqa: F401
 from . import fubapel  # noqa: F401
 from . import gerivik  # noqa: F401
+from . import zinesun  # noqa: F401

@@ -138,6 +138,16 @@ class Added:
         self.squares = squares
 
 
+class Averaged(Added):
+    """What a block hands on when the stream is complete and is a weighted average over the results of the blocks so
+    far: ``history`` float32 [total, N, H] holds those results (entry 0: the embedding's output), the first ``count``
+    of them are filled.  The next block of the kind appends its own."""
+
+    def __init__(self, history, count):
+        super().__init__(None)
+        self.history, self.count = history, int(count)
+
+
 class Normed:
     """The RMSNorm of the float32 residual stream, not computed yet.  ``added`` is what completed the stream
     (``Added``: nothing is pending for it, and its rows' sums of squares are there).  ``linear`` makes the norm
@@ -850,32 +860,39 @@ def sample(logits, temperatures, seeds, counters, out=None):
 
 # ---------------------------------------------------------------------------------------------------------------
 # Norms with a scaled residual add; gate functions by name
-def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0, bias=None):
     """stream += delta_scale * delta (in place, float32; skipped if delta is None); returns the norm of the sum as
-    out_dtype: layer norm without a bias (``centre``: the mean is removed, the variance is that of the centred row)
-    or RMS norm, times ``weight``, rounded once.  ``delta``: tensor of ``out_dtype`` [N, H] or Partials."""
+    out_dtype: layer norm (``centre``: the mean is removed, the variance is that of the centred row) or RMS norm,
+    times ``weight``, plus ``bias`` (float32 [H]) if given, rounded once.  ``delta``: tensor of ``out_dtype`` [N, H]
+    or Partials."""
+    delta = _plain_delta(delta)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, (width,))
     pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
     out = torch.empty((n, width), dtype=out_dtype, device=stream.device)
     _check(library.load().qil_add_norm(_ptr(stream), pointer, code, splits, n, float(delta_scale), None, _ptr(weight),
-                                       _ptr(out), n, width, float(eps), 1, int(bool(centre)), _code(out_dtype), _stream()),
-           'add_norm')
+                                       _ptr(bias), _ptr(out), n, width, float(eps), 1, int(bool(centre)), _code(out_dtype),
+                                       _stream()), 'add_norm')
     return out
 
 
-def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0, bias=None):
     """``add_norm`` of the selected rows only, [len(rows), H]; stream is left as it is."""
+    delta = _plain_delta(delta)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, (width,))
     _require(rows, 'rows', torch.int32)
     pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
     out = torch.empty((rows.shape[0], width), dtype=out_dtype, device=stream.device)
     _check(library.load().qil_add_norm(_ptr(stream), pointer, code, splits, n, float(delta_scale), _ptr(rows), _ptr(weight),
-                                       _ptr(out), rows.shape[0], width, float(eps), 0, int(bool(centre)), _code(out_dtype),
-                                       _stream()), 'rows_norm')
+                                       _ptr(bias), _ptr(out), rows.shape[0], width, float(eps), 0, int(bool(centre)),
+                                       _code(out_dtype), _stream()), 'rows_norm')
     return out
 
 
@@ -897,15 +914,93 @@ def gated_act(gate_up, out_dtype, *, activation, limit=0.0, alpha=1.0, interleav
     return out
 
 
+# Activations of feed-forwards without a gate branch: name -> code of the kernel.  'xielu' (two stored numbers p, q):
+# z > 0: softplus(p) z^2 + z / 2, else (1 / 2 + softplus(q)) (exp(z) - 1 - z) + z / 2.  'gelu_tanh': the tanh form of gelu.
+PLAIN_ACTIVATIONS = {'xielu': 0, 'gelu_tanh': 1}
+
+
+def plain_act(x, out_dtype, *, activation, params=None):
+    """[N, I] (tensor of the model's type or Partials) -> act(x) [N, I] of ``out_dtype``, for an activation of
+    ``PLAIN_ACTIVATIONS``; ``params`` float32 [2]: the two stored numbers of 'xielu'.  float32 arithmetic, one rounding."""
+    n, inner = x.shape
+    pointer, code, splits = _operand(x, 'x', out_dtype, (n, inner))
+    if activation == 'xielu':
+        _require(params, 'params', torch.float32, (2,))
+    out = torch.empty((n, inner), dtype=out_dtype, device=x.device)
+    _check(library.load().qil_plain_act(pointer, code, splits, _ptr(out), n, inner, _code(out_dtype),
+                                        PLAIN_ACTIVATIONS[activation], _ptr(params), _stream()), 'plain_act')
+    return out
+
+
+def post_norm_scale_add(stream, value, *, weight, bias, channel_scale, eps, centre, out_dtype=None, history=None, depth=0,
+                        mix=None):
+    """A sub-layer's output joins the float32 residual stream as its norm: stream += channel_scale * (norm(value) *
+    weight + bias), in place and in float32 (``centre``: layer norm, else RMS norm; ``weight``, ``bias``,
+    ``channel_scale`` float32 [H] or None).  ``value``: a tensor of the model's type or float32, ``Partials`` or a
+    ``RoutedSum``.  With ``history`` (float32 [>= depth, N, H]) the sum X is stored as entry ``depth - 1`` and the
+    stream becomes sum_(j < depth) mix[j] * history[j], ``mix`` float32 [depth].  With ``out_dtype`` the new stream
+    comes back rounded to that type (what the next sub-layer's products read), else None."""
+    n, width = stream.shape
+    _require(stream, 'stream', torch.float32)
+    value = _plain_delta(value)
+    if isinstance(value, Partials):
+        _require(value.tensor, 'value', torch.float32, (value.splits, n, width))
+        pointer, code, splits = value.tensor.data_ptr(), 0, value.splits
+    else:
+        _require(value, 'value', None, (n, width))
+        pointer, code, splits = value.data_ptr(), _code(value.dtype), 1
+    for name, vector in (('weight', weight), ('bias', bias), ('channel_scale', channel_scale)):
+        if vector is not None:
+            _require(vector, name, torch.float32, (width,))
+    if depth:
+        _require(history, 'history', torch.float32)
+        _require(mix, 'mix', torch.float32, (depth,))
+        if history.ndim != 3 or history.shape[0] < depth or tuple(history.shape[1:]) != (n, width):
+            raise ValueError(f'post_norm_scale_add: history must be [>= {depth}, {n}, {width}]')
+    out = torch.empty((n, width), dtype=out_dtype, device=stream.device) if out_dtype is not None else None
+    _check(library.load().qil_post_norm_scale_add(_ptr(stream), pointer, code, splits, _ptr(weight), _ptr(bias),
+                                                  _ptr(channel_scale), float(eps), int(bool(centre)), _ptr(out),
+                                                  _code(out_dtype) if out_dtype is not None else 0,
+                                                  _ptr(history) if depth else None, int(depth),
+                                                  _ptr(mix) if depth else None, n, width, _stream()), 'post_norm_scale_add')
+    return out
+
+
+def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, out_dtype):
+    """x + conv(x): a causal convolution over time on every channel, conv(x)_t = sum_j weight[:, j] * x_(t - taps + 1 +
+    j), over the rows of every sequence of the step and the taps - 1 inputs before them, which are the sequence's
+    state (``state`` float32 [slots, taps - 1, H]: read unless the sequence starts at position 0, and left holding
+    the sequence's last taps - 1 inputs).  ``x`` float32 [N, H] (the residual stream), ``weight`` float32 [H, taps].
+    -> [N, H] of ``out_dtype``; float32 arithmetic, one rounding."""
+    n, width = x.shape
+    _require(x, 'x', torch.float32)
+    taps = weight.shape[1]
+    _require(weight, 'weight', torch.float32, (width, taps))
+    if taps > 1:
+        _require(state, 'state', torch.float32)
+        if state.ndim != 3 or tuple(state.shape[1:]) != (taps - 1, width):
+            raise ValueError(f'short_conv: state must be [slots, {taps - 1}, {width}]')
+    _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+    _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+    _require(seq_slots, 'seq_slots', torch.int32, (n_seqs,))
+    _require(row_seq, 'row_seq', torch.int32, (n,))
+    out = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    _check(library.load().qil_short_conv(_ptr(x), _ptr(weight), _ptr(state) if taps > 1 else None, _ptr(cu_seqlens),
+                                         _ptr(seq_starts), _ptr(seq_slots), _ptr(row_seq), _ptr(out), _code(out_dtype), n,
+                                         width, taps, _stream()), 'short_conv')
+    return out
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # Attention over a cached latent
 def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequencies, positions, slots, latent, rope,
-                   dtype):
-    """From the stacked down products ``down`` [N, q_rank + rank + rot] (tensor of ``dtype`` or Partials): the
-    RMS-normed query latent [N, q_rank] (returned); the RMS-normed key/value latent and the rotated shared key part go
-    into the caches ``latent`` [.., rank] / ``rope`` [.., rot] at ``slots`` (None: nothing is stored)."""
+                   dtype, gates=0):
+    """From the stacked down products ``down`` [N, q_rank + rank + rot (+ gates)] (tensor of ``dtype`` or Partials):
+    the RMS-normed query latent [N, q_rank] (returned); the RMS-normed key/value latent and the rotated shared key
+    part go into the caches ``latent`` [.., rank] / ``rope`` [.., rot] at ``slots`` (None: nothing is stored).  With
+    ``gates`` more columns the result is (query latent, float32 [N, gates] of their sigmoids)."""
     n = down.shape[0]
-    pointer, code, splits = _operand(down, 'down', dtype, (n, q_rank + rank + rot))
+    pointer, code, splits = _operand(down, 'down', dtype, (n, q_rank + rank + rot + gates))
     _require(q_weight, 'q_weight', torch.float32, (q_rank,))
     _require(c_weight, 'c_weight', torch.float32, (rank,))
     _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
@@ -917,10 +1012,12 @@ def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequenc
         if latent.shape[-1] != rank or rope.shape[-1] != rot or latent.shape[:-1] != rope.shape[:-1]:
             raise ValueError('latent_prepare: caches must be [.., rank] and [.., rot] over the same slots')
     out = torch.empty((n, q_rank), dtype=dtype, device=down.device)
+    gate = torch.empty((n, gates), dtype=torch.float32, device=down.device) if gates else None
     _check(library.load().qil_latent_prepare(pointer, code, splits, _ptr(q_weight), _ptr(c_weight), _ptr(frequencies),
-                                             _ptr(positions), _ptr(slots), _ptr(out), _ptr(latent), _ptr(rope), n, q_rank,
-                                             rank, rot, float(eps), _code(dtype), _stream()), 'latent_prepare')
-    return out
+                                             _ptr(positions), _ptr(slots), _ptr(out), _ptr(latent), _ptr(rope), _ptr(gate),
+                                             n, q_rank, rank, rot, gates, float(eps), _code(dtype), _stream()),
+           'latent_prepare')
+    return (out, gate) if gates else out
 
 
 HEAD_PRODUCT_BLAS_ROWS = 256     # rows from which a bfloat16 product per head goes to the GPU BLAS in one batch
@@ -979,12 +1076,14 @@ LATENT_KEY_PARTS = None     # tests: (keys a part, parts) forces the matrix-core
 
 
 def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot,
-                     cu_seqlens=None, seq_starts=None, n_seqs=None, max_query=None, max_context=None):
+                     cu_seqlens=None, seq_starts=None, n_seqs=None, max_query=None, max_context=None, window=None,
+                     gate=None):
     """Every row's attention over its request's cached latents: ``q`` float32 [N, heads * (rank + rot)] as
     ``latent_query`` makes it; caches [pages, page_size, rank] and [pages, page_size, rot]; row n sees keys
     j <= positions[n] of sequence row_seq[n] (a row of ``block_tables``).  ``sink`` float32 [heads] or None: a logit
-    per head that counts once in the softmax's denominator and has no value.  -> float32 [N, heads * rank], the
-    weighted sums of the latents.
+    per head that counts once in the softmax's denominator and has no value.  ``window`` w: the row at position p sees
+    the keys j with 0 <= p - j < w only.  ``gate`` float32 [N, heads]: a factor on every head's result.
+    -> float32 [N, heads * rank], the weighted sums of the latents.
 
     With the step's description (``cu_seqlens``, ``seq_starts``, ``n_seqs``, ``max_query``, ``max_context``; rows packed
     sequence after sequence) bfloat16 caches of sizes it takes go to the matrix-core kernel, which serves several rows
@@ -1001,6 +1100,11 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
     _require(positions, 'positions', torch.int32, (n,))
     if sink is not None:
         _require(sink, 'sink', torch.float32, (heads,))
+    if gate is not None:
+        _require(gate, 'gate', torch.float32, (n, heads))
+    if window is not None and (type(window) is not int or window < 1):
+        raise ValueError('latent_attention: a window is a positive integer')
+    window = window or 0
     lib = library.load()
     if not lib.qil_latent_attention_takes(heads, rank, rot):
         raise UnsupportedShape(f'latent attention: {heads} heads, rank {rank}, {rot} rotated elements')
@@ -1013,20 +1117,20 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
             raise ValueError('one block table row per sequence, wide enough for the longest context')
         single = int(max_query == 1)
         plan = [ctypes.c_int(0) for _ in range(4)]
-        lib.qil_latent_mfma_plan(n, n_seqs, single, heads, max_context, *[ctypes.byref(v) for v in plan])
+        lib.qil_latent_mfma_plan(n, n_seqs, single, heads, max_context, window, *[ctypes.byref(v) for v in plan])
         rt, hb, part, parts = (v.value for v in plan)
         if LATENT_KEY_PARTS is not None:
             part, parts = LATENT_KEY_PARTS[0], max(LATENT_KEY_PARTS[1], -(-max_context // LATENT_KEY_PARTS[0]))
         nbytes = lib.qil_latent_mfma_workspace(n, heads, rank, parts)
         workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=q.device) if nbytes else None
         _check(lib.qil_latent_mfma(_ptr(q), _ptr(latent), _ptr(rope), _ptr(block_tables), block_tables.shape[1],
-                                   _ptr(cu_seqlens), _ptr(seq_starts), _ptr(positions), _ptr(sink), _ptr(out),
-                                   _ptr(workspace), n, n_seqs, single, heads, rank, rot, page_size, float(scale), rt, hb,
-                                   part, parts, _stream()), 'latent_mfma')
+                                   _ptr(cu_seqlens), _ptr(seq_starts), _ptr(positions), _ptr(sink), _ptr(gate), _ptr(out),
+                                   _ptr(workspace), n, n_seqs, single, heads, rank, rot, page_size, float(scale), window,
+                                   rt, hb, part, parts, _stream()), 'latent_mfma')
         return out
     _check(lib.qil_latent_attention(_ptr(q), _ptr(latent), _ptr(rope), _ptr(block_tables), block_tables.shape[1],
-                                    _ptr(row_seq), _ptr(positions), _ptr(sink), _ptr(out), n, heads, rank, rot, page_size,
-                                    float(scale), _code(latent.dtype), _stream()), 'latent_attention')
+                                    _ptr(row_seq), _ptr(positions), _ptr(sink), _ptr(gate), _ptr(out), n, heads, rank, rot,
+                                    page_size, float(scale), window, _code(latent.dtype), _stream()), 'latent_attention')
     return out
 
 
@@ -1131,24 +1235,27 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
 
 # ---------------------------------------------------------------------------------------------------------------
 # Routed feed-forward
-def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None):
     """x [N, width] (model type), router float32 [outputs, width], correction float32 [outputs] or None ->
     (chosen int32 [N, top], weights float32 [N, top]): softmax scores over all outputs in float32; the choice goes
     by score + correction among the outputs of the ``keep`` best of ``groups`` equal groups of neighbours (a group's
-    score: its best choice score); the weights are the chosen outputs' scores (divided by their sum if asked)."""
+    score: its best choice score); the weights are the chosen outputs' scores (divided by their sum if asked, which
+    makes them the softmax over the chosen logits alone).  ``bias`` float32 [outputs]: added to the logits."""
     n, width = x.shape
     _require(x, 'x')
     outputs = router.shape[0]
     _require(router, 'router', torch.float32, (outputs, width))
     if correction is not None:
         _require(correction, 'correction', torch.float32, (outputs,))
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, (outputs,))
     lib = library.load()
     if not lib.qil_moe_takes(width, outputs, 0, groups, keep, top):
         raise UnsupportedShape(f'moe_route: {outputs} outputs in {groups} groups ({keep} kept), top {top}, width {width}')
     chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=x.device)
     logits = torch.empty((n, outputs), dtype=torch.float32, device=x.device)
-    _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(correction), _ptr(logits), _ptr(chosen),
+    _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(bias), _ptr(correction), _ptr(logits), _ptr(chosen),
                              _ptr(weights), n, width, outputs, groups, keep, top, int(bool(renormalize)), _stream()),
            'moe_route')
     return chosen, weights

@@ -287,22 +287,22 @@ def _declare(lib):
     lib.qil_gemm_bf16_wide_gated_takes.argtypes = [i, i, i]
     lib.qil_gemm_bf16_wide_gated_takes.restype = i
     lib.qil_gemm_bf16_wide_gated.argtypes = [p, p, p, i, i, i, i, p]
-    lib.qil_add_norm.argtypes = [p, p, i, i, i, f, p, p, p, i, i, f, i, i, i, p]
+    lib.qil_add_norm.argtypes = [p, p, i, i, i, f, p, p, p, p, i, i, f, i, i, i, p]
     lib.qil_gated_act.argtypes = [p, i, i, p, i, i, i, i, i, f, f, p]
-    lib.qil_latent_prepare.argtypes = [p, i, i, p, p, p, p, p, p, p, p, i, i, i, i, f, i, p]
+    lib.qil_latent_prepare.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, f, i, p]
     lib.qil_head_product.argtypes = [p, i, i, i, p, i, p, i, i, i, i, i, i, i, p]
     lib.qil_rotate_tail.argtypes = [p, i, i, i, i, p, p, p, i, i, i, i, i, i, p]
     lib.qil_latent_attention_takes.argtypes = [i, i, i]
     lib.qil_latent_attention_takes.restype = i
-    lib.qil_latent_attention.argtypes = [p, p, p, p, i, p, p, p, p, i, i, i, i, i, f, i, p]
+    lib.qil_latent_attention.argtypes = [p, p, p, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, p]
     lib.qil_latent_mfma_takes.argtypes = [i, i, i]
     lib.qil_latent_mfma_takes.restype = i
     ip = ctypes.POINTER(ctypes.c_int)
-    lib.qil_latent_mfma_plan.argtypes = [i, i, i, i, i, ip, ip, ip, ip]
+    lib.qil_latent_mfma_plan.argtypes = [i, i, i, i, i, i, ip, ip, ip, ip]
     lib.qil_latent_mfma_plan.restype = None
     lib.qil_latent_mfma_workspace.argtypes = [i, i, i, i]
     lib.qil_latent_mfma_workspace.restype = z
-    lib.qil_latent_mfma.argtypes = [p, p, p, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, i, i, p]
+    lib.qil_latent_mfma.argtypes = [p, p, p, p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, i, i, i, p]
     lib.qil_latent_mfma.restype = i
     lib.qil_state_scan_slot.argtypes = [i, i, i, i]
     lib.qil_state_scan_slot.restype = z
@@ -325,7 +325,7 @@ def _declare(lib):
     lib.qil_moe_combine.restype = i
     lib.qil_moe_takes.argtypes = [i, i, i, i, i, i]
     lib.qil_moe_takes.restype = i
-    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_moe_route.restype = i
     lib.qil_moe_tile_rows.argtypes = [i, i]
     lib.qil_moe_tile_rows.restype = i
@@ -333,6 +333,12 @@ def _declare(lib):
     lib.qil_moe_max_tiles.restype = i
     lib.qil_moe_experts.argtypes = [p, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, f, p]
     lib.qil_moe_experts.restype = i
+    lib.qil_post_norm_scale_add.argtypes = [p, p, i, i, p, p, p, f, i, p, i, p, i, p, i, i, p]
+    lib.qil_post_norm_scale_add.restype = i
+    lib.qil_short_conv.argtypes = [p, p, p, p, p, p, p, p, i, i, i, i, p]
+    lib.qil_short_conv.restype = i
+    lib.qil_plain_act.argtypes = [p, i, i, p, i, i, i, i, p, p]
+    lib.qil_plain_act.restype = i
     lib.qil_sample.argtypes = [p, p, p, p, p, p, p, i, i, p]
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z

@@ -1,18 +1,20 @@
 """Parts that models are assembled from."""
-from .base import (ParamSpec, KVNeed, PagedNeed, StateNeed, Part, Norm, PositionEncoding, Rotation,
+from .base import (ParamSpec, KVNeed, PagedNeed, StateNeed, CompoundNeed, Part, Norm, PositionEncoding, Rotation,
                    Mixer, FeedForward, Block)
 from .norm import RMSNorm, LayerNorm
 from .rotary import Rotary, RotaryFrequencies
 from .attention import Attention
 from .latent_attention import LatentAttention
 from .recurrent import MatrixMemory
-from .mlp import GatedMLP
+from .mlp import GatedMLP, PlainMLP
+from .conv import ShortConvolution
 from .moe import RoutedExperts
-from .block import PreNormBlock, SandwichBlock
+from .block import PreNormBlock, SandwichBlock, PostNormBlock
 from .embedding import Embedding, LMHead
 from .model import CausalLM, ScheduleEntry
 
-__all__ = ['ParamSpec', 'KVNeed', 'PagedNeed', 'StateNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
+__all__ = ['ParamSpec', 'KVNeed', 'PagedNeed', 'StateNeed', 'CompoundNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
            'FeedForward', 'Block', 'RMSNorm', 'LayerNorm', 'Rotary', 'RotaryFrequencies', 'Attention',
-           'LatentAttention', 'MatrixMemory', 'GatedMLP', 'RoutedExperts', 'PreNormBlock', 'SandwichBlock',
+           'LatentAttention', 'MatrixMemory', 'GatedMLP', 'PlainMLP', 'ShortConvolution', 'RoutedExperts', 'PreNormBlock',
+           'SandwichBlock', 'PostNormBlock',
            'Embedding', 'LMHead', 'CausalLM', 'ScheduleEntry']

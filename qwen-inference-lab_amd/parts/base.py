@@ -59,6 +59,14 @@ class StateNeed:
     dtype: str = 'float32'
 
 
+@dataclass(frozen=True)
+class CompoundNeed:
+    """Several needs of one schedule entry: ``needs`` is a tuple of KVNeed | PagedNeed | StateNeed (a block whose
+    mixer keeps pages while another of its parts keeps a fixed-size state).  Each need joins the group of its kind as
+    if it stood alone; the entry's view is the tuple of their views, in the same order."""
+    needs: tuple
+
+
 class Part:
     def __init__(self):
         self.p = {}
@@ -172,6 +180,11 @@ class Block(Part):
     def parts(self):
         """dict local prefix -> Part (for naming tensors)."""
         return {}
+
+    def cache_need(self):
+        """What a run of the block keeps between steps: its mixer's need, unless the block has parts of its own
+        that keep something too (then a ``CompoundNeed``, and ``forward`` gets the tuple of views)."""
+        return self.mixer.cache_need() if self.mixer is not None else None
 
     def forward(self, stream, pending, ctx, cache):
         raise NotImplementedError

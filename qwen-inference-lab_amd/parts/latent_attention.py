@@ -18,11 +18,20 @@ class LatentAttention(Mixer):
     Keys and values are never expanded: the query is multiplied by W_uk,h^T once (``ops.latent_query``), the
     attention kernel works on the cached rows themselves, and W_uv,h is applied to the weighted sum of latents.
     ``position``: a ``RotaryFrequencies`` over ``rot_dim`` elements.
+    ``window`` w: row i sees the keys j with 0 <= i - j < w only, and the cache gives pages back that no later row
+    sees (None: every key j <= i).
+    ``gate``: head h's result is multiplied by sigmoid(W_g x)_h (tensor ``g_proj.weight`` [heads, width]; the
+    sigmoid in float32); W_g is stacked under the two down projections, so the gate costs no product of its own.
+    ``pairing``: which elements of the rotated parts a rotation pairs: 'halves', (i, i + rot_dim / 2), which is what
+    the kernels do, or 'neighbours', (2 i, 2 i + 1) with the same frequency f_i.  A score does not change when the
+    elements of the query's and the key's rotated part are reordered alike, so for 'neighbours' the rows of W_uq
+    (every head's rotated part) and of W_dkv (the shared rotated part) are reordered once at ``finalize``, even
+    elements first, and the kernels run as they are.
     """
     graph_safe = True
 
     def __init__(self, *, width, heads, dim, rot_dim, vdim, kv_rank, q_rank, scale, eps, position, sink=True,
-                 dtype=torch.bfloat16):
+                 window=None, gate=False, pairing='halves', dtype=torch.bfloat16):
         super().__init__()
         for name, value in (('heads', heads), ('dim', dim), ('vdim', vdim), ('kv_rank', kv_rank), ('q_rank', q_rank)):
             if type(value) is not int or value < 1:
@@ -34,6 +43,11 @@ class LatentAttention(Mixer):
         self.width, self.heads, self.dim, self.rot_dim, self.vdim = width, heads, dim, rot_dim, vdim
         self.kv_rank, self.q_rank, self.scale, self.eps = kv_rank, q_rank, float(scale), float(eps)
         self.position, self.sink, self.dtype = position, bool(sink), dtype
+        if window is not None and (type(window) is not int or window < 1):
+            raise ops.UnsupportedShape(f'window must be a positive integer or None, not {window!r}')
+        if pairing not in ('halves', 'neighbours'):
+            raise ValueError(f"pairing must be 'halves' or 'neighbours', not {pairing!r}")
+        self.window, self.gate, self.pairing = window, bool(gate), pairing
 
     def param_specs(self):
         h, d, r = self.heads, self.dim, self.rot_dim
@@ -47,15 +61,25 @@ class LatentAttention(Mixer):
                  'o_proj.weight': ParamSpec((self.width, h * self.vdim))}
         if self.sink:
             specs['sink'] = ParamSpec((h,), 'vector', 'normal')
+        if self.gate:
+            specs['g_proj.weight'] = ParamSpec((h, self.width))
         return specs
 
     def cache_need(self):
-        return PagedNeed((('latent', (self.kv_rank,), 'model'), ('rope', (self.rot_dim,), 'model')), None)
+        return PagedNeed((('latent', (self.kv_rank,), 'model'), ('rope', (self.rot_dim,), 'model')), self.window)
 
     def finalize(self):
         p = self.p
-        # both down products in one: [q_rank + kv_rank + rot_dim, width]
-        self.w_down = torch.cat([p.pop('q_down.weight'), p.pop('kv_down.weight')]).contiguous()
+        if self.pairing == 'neighbours':                # even elements of every rotated part first: (2 i, 2 i + 1) -> (i, i + r / 2)
+            d, r = self.dim, self.rot_dim
+            order = torch.cat([torch.arange(0, r, 2), torch.arange(1, r, 2)]).to(p['q_up.weight'].device)
+            q_up = p['q_up.weight'].view(self.heads, d + r, self.q_rank)
+            p['q_up.weight'] = torch.cat([q_up[:, :d], q_up[:, d:][:, order]], dim=1).reshape(-1, self.q_rank).contiguous()
+            kv_down = p['kv_down.weight']
+            p['kv_down.weight'] = torch.cat([kv_down[:self.kv_rank], kv_down[self.kv_rank:][order]]).contiguous()
+        # the down products in one: [q_rank + kv_rank + rot_dim (+ heads), width]
+        stacked = [p.pop('q_down.weight'), p.pop('kv_down.weight')] + ([p.pop('g_proj.weight')] if self.gate else [])
+        self.w_down = torch.cat(stacked).contiguous()
         p['down.weight'] = self.w_down
         # W_uk as [heads, dim, kv_rank] is the layout the query's product reads (a pure view); W_uv per head transposed
         self.k_up = p['k_up.weight'].view(self.heads, self.dim, self.kv_rank)
@@ -69,7 +93,9 @@ class LatentAttention(Mixer):
         cq = ops.latent_prepare(down, q_rank=self.q_rank, rank=self.kv_rank, rot=self.rot_dim, q_weight=p['q_norm.weight'],
                                 c_weight=p['kv_norm.weight'], eps=self.eps, frequencies=frequencies,
                                 positions=ctx.positions, slots=cache.slots if cache.writes else None,
-                                latent=cache.tensors['latent'], rope=cache.tensors['rope'], dtype=self.dtype)
+                                latent=cache.tensors['latent'], rope=cache.tensors['rope'], dtype=self.dtype,
+                                gates=self.heads if self.gate else 0)
+        cq, gate = cq if self.gate else (cq, None)
         q = ops.linear(cq, p['q_up.weight'], None)
         q = ops.latent_query(q, self.k_up, heads=self.heads, dim=self.dim, rot=self.rot_dim, rank=self.kv_rank,
                              frequencies=frequencies, positions=ctx.positions)
@@ -78,6 +104,6 @@ class LatentAttention(Mixer):
                                      positions=ctx.positions, sink=p.get('sink'), scale=self.scale, heads=self.heads,
                                      rank=self.kv_rank, rot=self.rot_dim, cu_seqlens=ctx.cu_seqlens,
                                      seq_starts=ctx.seq_starts, n_seqs=ctx.n_seqs, max_query=ctx.max_query,
-                                     max_context=ctx.max_context)
+                                     max_context=ctx.max_context, window=self.window, gate=gate)
         values = ops.head_product(mixed, p['v_up.weight'], heads=self.heads, out_dtype=self.dtype)
         return ops.linear(values, p['o_proj.weight'], None, partials=True)

@@ -1,4 +1,4 @@
-"""Gated feed-forward: down(act(gate(x)) * up(x)).  Formula: qil/model.py:71."""
+"""Feed-forwards: gated, down(act(gate(x)) * up(x)) (formula: qil/model.py:71), and plain, down(act(up(x)))."""
 import torch
 
 from .base import FeedForward, ParamSpec
@@ -39,4 +39,28 @@ class GatedMLP(FeedForward):
                                   activation=self.activation, limit=self.limit, alpha=self.alpha)
         if add_to is not None and hidden.is_cuda:              # few rows: the down product adds into the stream itself
             return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True, add_to=add_to)
+        return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)
+
+
+class PlainMLP(FeedForward):
+    """down(act(up(x))) without a gate branch and without biases.  ``activation`` names a function of
+    ``ops.PLAIN_ACTIVATIONS``; 'xielu' has two stored numbers (p, q), the tensor ``act``, and is
+    softplus(p) z^2 + z / 2 for z > 0, (1 / 2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise, in float32."""
+
+    def __init__(self, *, width, intermediate, activation='xielu', dtype=torch.bfloat16):
+        super().__init__()
+        if activation not in ops.PLAIN_ACTIVATIONS:
+            raise ValueError(f'no kernel for activation {activation!r}')
+        self.width, self.intermediate, self.activation, self.dtype = width, intermediate, activation, dtype
+
+    def param_specs(self):
+        specs = {'up_proj.weight': ParamSpec((self.intermediate, self.width)),
+                 'down_proj.weight': ParamSpec((self.width, self.intermediate))}
+        if self.activation == 'xielu':
+            specs['act'] = ParamSpec((2,), 'vector', 'normal')
+        return specs
+
+    def forward(self, h):
+        hidden = ops.plain_act(ops.linear(h, self.p['up_proj.weight'], None, partials=True), self.dtype,
+                               activation=self.activation, params=self.p.get('act'))
         return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

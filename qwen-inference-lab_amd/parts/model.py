@@ -3,7 +3,7 @@ from dataclasses import dataclass
 
 import torch
 
-from .base import KVNeed, PagedNeed, StateNeed
+from .base import KVNeed, PagedNeed, StateNeed, CompoundNeed
 from .. import ops
 
 
@@ -52,8 +52,7 @@ class CausalLM:
         self.loaded = False
 
     def _need(self, entry):
-        mixer = self.blocks[entry.block].mixer
-        return mixer.cache_need() if mixer is not None else None
+        return self.blocks[entry.block].cache_need()
 
     def all_parts(self):
         seen, out = set(), []
@@ -71,11 +70,12 @@ class CausalLM:
         return out
 
     def cache_needs(self):
-        """Per schedule entry: KVNeed | PagedNeed | StateNeed | None, or ('shared', owner position)."""
+        """Per schedule entry: KVNeed | PagedNeed | StateNeed | CompoundNeed | None, or ('shared', owner position)."""
         needs = []
         for entry in self.schedule:
             need = self._need(entry)
-            if need is not None and not isinstance(need, (KVNeed, PagedNeed, StateNeed)):
+            single = need.needs if isinstance(need, CompoundNeed) else (need,)
+            if need is not None and not all(isinstance(one, (KVNeed, PagedNeed, StateNeed)) for one in single):
                 raise TypeError(f'unknown cache need {need!r}')
             needs.append(need if entry.cache_of is None or need is None else ('shared', entry.cache_of))
         return needs

@@ -10,10 +10,11 @@ class RoutedExperts(FeedForward):
     which every token uses ``top``, and ``identity`` more router outputs that stand for experts without tensors whose
     output is their input.
 
-    Router: logits over experts + identity outputs in float32 (the router matrix stays float32 in every model),
-    softmax over all of them; the choice goes by score + ``correction`` (a stored vector, if ``correction``) among the
+    Router: logits over experts + identity outputs in float32 (the router matrix stays float32 in every model), plus
+    a stored bias per output if ``bias``; softmax over all of them; the choice goes by score + ``correction`` (a stored vector, if ``correction``) among the
     outputs of the ``keep`` best of ``groups`` equal groups of neighbouring outputs, a group's score being its best
-    choice score; the weights are the chosen outputs' softmax scores, divided by their sum only if ``renormalize``.
+    choice score; the weights are the chosen outputs' softmax scores, divided by their sum only if ``renormalize``
+    (which makes them the softmax over the chosen logits alone).
     The result is the weighted sum of the chosen experts' outputs, in float32.
 
     The experts' matrices are stacked at ``finalize`` into [experts, 2, ff, width] (gate rows, then up rows) and
@@ -22,7 +23,7 @@ class RoutedExperts(FeedForward):
     """
 
     def __init__(self, *, width, experts, identity=0, top, groups=1, keep=1, intermediate, activation='silu', limit=None,
-                 alpha=1.0, correction=False, renormalize=False, dtype=torch.bfloat16):
+                 alpha=1.0, correction=False, renormalize=False, bias=False, dtype=torch.bfloat16):
         super().__init__()
         for name, value in (('experts', experts), ('top', top), ('groups', groups), ('keep', keep),
                             ('intermediate', intermediate)):
@@ -40,10 +41,12 @@ class RoutedExperts(FeedForward):
         self.width, self.experts, self.identity, self.top, self.groups, self.keep = width, experts, identity, top, groups, keep
         self.outputs, self.intermediate, self.activation = outputs, intermediate, activation
         self.limit, self.alpha, self.correction, self.renormalize = float(limit or 0.0), float(alpha), bool(correction), bool(renormalize)
-        self.dtype = dtype
+        self.dtype, self.bias = dtype, bool(bias)
 
     def param_specs(self):
         specs = {'router.weight': ParamSpec((self.outputs, self.width), 'vector')}
+        if self.bias:
+            specs['router.bias'] = ParamSpec((self.outputs,), 'vector')
         if self.correction:
             specs['router.correction'] = ParamSpec((self.outputs,), 'vector')
         for e in range(self.experts):
@@ -67,7 +70,7 @@ class RoutedExperts(FeedForward):
     def forward(self, h, add_to=None):
         p = self.p
         chosen, weights = ops.moe_route(h, p['router.weight'], p.get('router.correction'), groups=self.groups,
-                                        keep=self.keep, top=self.top, renormalize=self.renormalize)
+                                        keep=self.keep, top=self.top, renormalize=self.renormalize, bias=p.get('router.bias'))
         out = ops.moe_experts(h, chosen, weights, p['experts.gate_up_proj.weight'], p['experts.down_proj.weight'],
                               activation=self.activation, limit=self.limit, alpha=self.alpha, lazy=True)
         if isinstance(out, ops.RoutedSum):              # the norm that follows makes the weighted sum as it loads the rows

@@ -1,4 +1,4 @@
-"""Norms with float32 statistics: RMSNorm (formula: qil/model.py:15-23) and a layer norm without a bias."""
+"""Norms with float32 statistics: RMSNorm (formula: qil/model.py:15-23) and a layer norm with or without a bias."""
 import torch
 
 from .base import Norm, ParamSpec
@@ -7,6 +7,7 @@ from .. import ops
 
 class RMSNorm(Norm):
     """y = cast(x * rsqrt(mean(x^2) + eps)) * weight; weight multiplies as stored."""
+    centre = False
 
     def __init__(self, width, eps):
         super().__init__()
@@ -33,19 +34,24 @@ class RMSNorm(Norm):
 
 
 class LayerNorm(Norm):
-    """y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight: a weight, no bias; float32 throughout and one
+    """y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight (+ bias, if ``bias``); float32 throughout and one
     rounding of the result.  ``delta_scale`` multiplies the sub-layer output that is added into the stream first."""
+    centre = True
 
-    def __init__(self, width, eps):
+    def __init__(self, width, eps, bias=False):
         super().__init__()
-        self.width, self.eps = int(width), float(eps)
+        self.width, self.eps, self.bias = int(width), float(eps), bool(bias)
 
     def param_specs(self):
-        return {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal')}
+        specs = {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal')}
+        if self.bias:
+            specs['bias'] = ParamSpec((self.width,), 'vector', 'normal')
+        return specs
 
     def forward(self, stream, delta, out_dtype, delta_scale=1.0):
-        return ops.add_norm(stream, delta, self.p['weight'], self.eps, out_dtype, centre=True, delta_scale=delta_scale)
+        return ops.add_norm(stream, delta, self.p['weight'], self.eps, out_dtype, centre=True, delta_scale=delta_scale,
+                            bias=self.p.get('bias'))
 
     def forward_rows(self, stream, delta, rows, out_dtype, delta_scale=1.0):
         return ops.rows_norm(stream, delta, rows, self.p['weight'], self.eps, out_dtype, centre=True,
-                             delta_scale=delta_scale)
+                             delta_scale=delta_scale, bias=self.p.get('bias'))
