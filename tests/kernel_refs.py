@@ -181,17 +181,62 @@ def _any_norm(x, weight, eps, centre):
     return x / torch.sqrt(x.square().mean(dim=-1, keepdim=True) + eps) * weight
 
 
-def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0, bias=None):
     if delta is not None:
         stream += delta_scale * _value(delta).to(torch.float32)
-    return _any_norm(stream, weight, eps, centre).to(out_dtype)
+    return (_any_norm(stream, weight, eps, centre) + (bias if bias is not None else 0.0)).to(out_dtype)
 
 
-def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0, bias=None):
     x = stream[rows.long()]
     if delta is not None:
         x = x + delta_scale * _value(delta)[rows.long()].to(torch.float32)
-    return _any_norm(x, weight, eps, centre).to(out_dtype)
+    return (_any_norm(x, weight, eps, centre) + (bias if bias is not None else 0.0)).to(out_dtype)
+
+
+def plain_act(x, out_dtype, *, activation, params=None):
+    z = _value(x).to(torch.float32)
+    if activation == 'gelu_tanh':
+        return (0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))).to(out_dtype)
+    soft = torch.nn.functional.softplus(params)
+    below = z.clamp(max=0.0)
+    return torch.where(z > 0, soft[0] * z * z + 0.5 * z, (0.5 + soft[1]) * (torch.expm1(below) - below) + 0.5 * z).to(out_dtype)
+
+
+def post_norm_scale_add(stream, value, *, weight, bias, channel_scale, eps, centre, out_dtype=None, history=None, depth=0,
+                        mix=None):
+    y = _value(value).to(torch.float32)
+    if centre:
+        y = y - y.mean(dim=-1, keepdim=True)
+    z = y / torch.sqrt(y.square().mean(dim=-1, keepdim=True) + eps)
+    if weight is not None:
+        z = z * weight
+    if bias is not None:
+        z = z + bias
+    if channel_scale is not None:
+        z = z * channel_scale
+    stream += z
+    if depth:
+        history[depth - 1] = stream
+        stream.copy_((mix[:depth, None, None] * history[:depth]).sum(dim=0))
+    return stream.to(out_dtype) if out_dtype is not None else None
+
+
+def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, out_dtype):
+    taps, keep = weight.shape[1], weight.shape[1] - 1
+    out = torch.empty_like(x)
+    for s in range(n_seqs):
+        first, last, start = int(cu_seqlens[s]), int(cu_seqlens[s + 1]), int(seq_starts[s])
+        before = torch.zeros((keep, x.shape[1]), dtype=torch.float32)
+        if keep and start > 0:
+            before = state[int(seq_slots[s])].clone()
+            before[:max(0, keep - start)] = 0.0                 # places before the sequence's start
+        inputs = torch.cat([before, x[first:last]])
+        for t in range(last - first):
+            out[first + t] = x[first + t] + (weight.t() * inputs[t:t + taps]).sum(dim=0)
+        if keep:
+            state[int(seq_slots[s])] = inputs[-keep:]
+    return out.to(out_dtype)
 
 
 def gated_act(gate_up, out_dtype, *, activation, limit=0.0, alpha=1.0, interleaved=False):
@@ -210,13 +255,13 @@ def _turn(x, positions, frequencies):
 
 
 def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequencies, positions, slots, latent, rope,
-                   dtype):
+                   dtype, gates=0):
     x = _value(down).to(torch.float32)
     cq = _any_norm(x[:, :q_rank], q_weight, eps, False).to(dtype)
     if slots is not None:
         latent.view(-1, rank)[slots.long()] = _any_norm(x[:, q_rank:q_rank + rank], c_weight, eps, False).to(dtype)
-        rope.view(-1, rot)[slots.long()] = _turn(x[:, q_rank + rank:], positions, frequencies).to(dtype)
-    return cq
+        rope.view(-1, rot)[slots.long()] = _turn(x[:, q_rank + rank:q_rank + rank + rot], positions, frequencies).to(dtype)
+    return (cq, torch.sigmoid(x[:, q_rank + rank + rot:])) if gates else cq
 
 
 def head_product(x, weight, *, heads, out_dtype, out=None, out_columns=None):
@@ -236,13 +281,14 @@ def latent_query(q, k_up, *, heads, dim, rot, rank, frequencies, positions):
 
 
 def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot,
-                     **step):
+                     window=None, gate=None, **step):
     n = q.shape[0]
     q = q.view(n, heads, rank + rot)
     out = torch.zeros((n, heads, rank), dtype=torch.float32)
     flat_c, flat_r = latent.view(-1, rank).to(torch.float32), rope.view(-1, rot).to(torch.float32)
     for row in range(n):
-        keys = torch.arange(int(positions[row]) + 1)
+        place = int(positions[row])
+        keys = torch.arange(max(0, place - window + 1) if window else 0, place + 1)
         table = block_tables[int(row_seq[row])].long()
         slots = table[keys // page_size] * page_size + keys % page_size
         c, r = flat_c[slots], flat_r[slots]
@@ -251,6 +297,8 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
             scores = torch.cat([scores, sink[:, None]], dim=1)
         p = torch.softmax(scores, dim=1)[:, :len(keys)]
         out[row] = p @ c
+        if gate is not None:
+            out[row] *= gate[row, :, None]
     return out.reshape(n, heads * rank)
 
 
@@ -327,9 +375,10 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
     return (unit * (torch.sigmoid(g) if gate == 'sigmoid' else g * torch.sigmoid(g))).to(out_dtype)
 
 
-def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
-    scores = torch.softmax(x.to(torch.float32) @ router.t(), dim=-1)
-    choice = scores + correction if correction is not None else scores.clone()
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None):
+    logits = x.to(torch.float32) @ router.t() + (bias if bias is not None else 0.0)
+    scores = torch.softmax(logits, dim=-1)
+    choice = scores + correction if correction is not None else logits.clone()
     n, outputs = scores.shape
     if groups > 1 and keep < groups:
         best = choice.view(n, groups, outputs // groups).max(dim=-1).values
@@ -364,4 +413,4 @@ ALL = dict(moe_route=moe_route, moe_experts=moe_experts, embed=embed, add_rmsnor
            qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample,
            add_norm=add_norm, rows_norm=rows_norm, gated_act=gated_act, latent_prepare=latent_prepare, head_product=head_product,
            latent_query=latent_query, latent_attention=latent_attention, state_scan_slot=state_scan_slot, state_scan=state_scan,
-           head_norm_gate=head_norm_gate)
+           head_norm_gate=head_norm_gate, plain_act=plain_act, post_norm_scale_add=post_norm_scale_add, short_conv=short_conv)
