@@ -3,5 +3,6 @@ from .base import ConfigError, read_config_json
 from .qwen3 import Qwen3Config
 from .fubapel import FubapelConfig
 from .gerivik import GerivikConfig
+from .zinesun import ZinesunConfig
 
-__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig', 'GerivikConfig']
+__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig', 'GerivikConfig', 'ZinesunConfig']
