@@ -238,6 +238,21 @@ def gerivik_config(z, layers, vocab):
                 layers=[kinds[i % 2] for i in range(layers)], norm=dict(eps=1e-6))
 
 
+def zinesun_config(z, layers, vocab, window, kind='turns'):
+    """`layers` layers of windowed latent attention at the sizes of Fubapel's, a four-tap convolution in front of each;
+    behind them a dense xielu feed-forward one and a half times as wide as the gated ones beside it (two matrices
+    instead of three: equal weights and arithmetic), or a routed one (32 experts of a quarter of the gated
+    feed-forward's inner size, 4 chosen: a token's experts are as large as the gated one), or both in turns."""
+    mixer = dict(heads=z['heads'], dim=z['dim'], rot_dim=z['rot_dim'], vdim=z['dim'], kv_rank=z['kv_rank'], q_rank=z['q_rank'],
+                 rot=dict(base=10000.0, dims=z['rot_dim']), scale=(z['dim'] + z['rot_dim']) ** -0.5, mask=dict(size=window))
+    dense = dict(kind='dense', ff=z['ff'] * 3 // 2)
+    routed = dict(kind='moe', expert=dict(ff=z['ff'] // 4), router=dict(experts=32, top=4))
+    feeds = dict(turns=[dense, routed], dense=[dense], routed=[routed])[kind]
+    return dict(architecture='Zinesun', vocab=vocab, width=z['width'], embedding=dict(scale=z['width'] ** 0.5), canon=dict(taps=4),
+                layers=[dict(type='latent_attention', mixer=mixer, mlp=feeds[i % len(feeds)]) for i in range(layers)],
+                norm=dict(eps=1e-5))
+
+
 def designs_phase(args, torch, dtype):
     """Prefill tokens a second and decode milliseconds a step of a design's models whose layers are all of one kind
     (and of its kinds in turns), beside dense Qwen3 of the same width, feed-forward, depth and attention heads."""
@@ -245,7 +260,15 @@ def designs_phase(args, torch, dtype):
     from qil_amd.engine import ModelRunner, StepEntry
     z, layers, vocab, page_size = DESIGN_SIZES[args.design_sizes], args.layers or 6, 32768, 16
     generator = torch.Generator().manual_seed(99)
-    if args.design == 'gerivik':
+    if args.design == 'zinesun':
+        # beside it the closest models of the engine: Fubapel's latent attention (no window, no gate, no convolution, a
+        # gated feed-forward, pre-norm) and Gerivik's capped attention with the routed feed-forward
+        models = {f'zinesun ({name}, window {args.design_window})': zinesun_config(z, layers, vocab, args.design_window, kind)
+                  for kind, name in (('turns', 'feed-forwards in turns'), ('dense', 'dense feed-forwards'), ('routed', 'routed feed-forwards'))}
+        models[f'zinesun (dense feed-forwards, window {8 * args.design_window})'] = zinesun_config(z, layers, vocab, 8 * args.design_window, 'dense')
+        models['fubapel (latent attention only)'] = dict(fubapel_config(z, layers, vocab), layers=[fubapel_config(z, 1, vocab)['layers'][0]] * layers)
+        models['gerivik (capped attention only)'] = dict(gerivik_config(z, layers, vocab), layers=[gerivik_config(z, 2, vocab)['layers'][1]] * layers)
+    elif args.design == 'gerivik':
         mixed = gerivik_config(z, layers, vocab)
         models = {'gerivik (kinds in turns)': mixed}
         for index, name in enumerate(('gated linear attention', 'capped attention')):
@@ -324,7 +347,8 @@ def main():
                              'attention kernels alone, at the reference\'s own shapes and at the benchmark\'s.  products: a layer\'s '
                              'matrix products at --prefill-tokens rows alone, GPU BLAS against own kernel.  designs: prefill and decode of the '
                              'design named by --design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
-    parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik'], help='the design of --phase designs')
+    parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik', 'zinesun'], help='the design of --phase designs')
+    parser.add_argument('--design-window', type=int, default=512, help='the attention window of --design zinesun')
     parser.add_argument('--design-sizes', default='1b', choices=sorted(DESIGN_SIZES), help='layer sizes of --phase designs')
     parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')
     parser.add_argument('--own-products', action='store_true',

@@ -361,9 +361,9 @@ void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max
   const long blocks = (long)tiles * ((heads + *hb - 1) / *hb);
   int want = (int)((2 * QIL_CUS + blocks - 1) / blocks);
   if (want < 1) want = 1;
-  int span = max_context;
-  if (window > 0 && window + *rt - 1 < span) span = window + *rt - 1;
-  int part = ((span + want - 1) / want + 31) / 32 * 32;
+  int span = max_context;                                     // what a block walks when it walks everything its rows see
+  if (want > 1 && window > 0 && window + *rt - 1 < span) span = window + *rt - 1;
+  int part = ((span + want - 1) / want + 31) / 32 * 32;      // (enough blocks: one part, and a block begins at its window)
   if (part < 64) part = 64;                                   // two steps a block: shorter parts cost more in the merge than they save
   *P = part;
   *parts = (max_context + part - 1) / part;
