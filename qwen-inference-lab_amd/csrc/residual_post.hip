@@ -10,49 +10,84 @@
 //
 // y: one array of the model's type or float32 partial sums [splits][rows][width]; everything else is float32.
 // One block per row; the row of y is held in LDS between the passes (statistics in two passes: the variance is that
-// of the deviations).
+// of the deviations); a thread takes four neighbouring elements at a time where the rows allow.
 #include "common.h"
 #include "partials.h"
 
-template <typename TD, typename T, int CENTRE>
+template <typename TD, typename T, int CENTRE, int V>
 __global__ void post_norm_scale_add_kernel(float* __restrict__ stream, const TD* __restrict__ y, int splits, size_t split_stride,
                                            const float* __restrict__ weight, const float* __restrict__ bias,
                                            const float* __restrict__ channel_scale, float eps, T* __restrict__ out,
                                            float* __restrict__ history, size_t history_stride, int depth,
                                            const float* __restrict__ mix, int width) {
-  extern __shared__ float row[];                      // [width]
+  extern __shared__ __align__(16) float row[];        // [width]
   __shared__ float scratch[16];
   const size_t at = (size_t)blockIdx.x * width;
+  const int step = blockDim.x * V;
   float sum = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = parts_sum(y, at + i, splits, split_stride);
-    row[i] = v;                                       // a thread rereads only what it wrote
-    sum += v;
+  for (int i = threadIdx.x * V; i < width; i += step) {          // a thread rereads only what it wrote
+    if (V == 4) {
+      float4 v = ld4(y + at + i);
+      for (int s = 1; s < splits; ++s) {
+        const float4 more = ld4(y + s * split_stride + at + i);
+        v.x += more.x, v.y += more.y, v.z += more.z, v.w += more.w;
+      }
+      st4(row + i, v);
+      sum += (v.x + v.y) + (v.z + v.w);
+    } else {
+      const float v = parts_sum(y, at + i, splits, split_stride);
+      row[i] = v;
+      sum += v;
+    }
   }
   float mean = 0.f;
   if (CENTRE) mean = block_sum(sum, scratch) / (float)width;
   float squares = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float c = row[i] - mean;
-    squares += c * c;
-  }
+  for (int i = threadIdx.x * V; i < width; i += step)
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float c = row[i + e] - mean;
+      squares += c * c;
+    }
   squares = block_sum(squares, scratch);
   const float scale = 1.f / sqrtf(squares / (float)width + eps);
   float* x = stream + at;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    float z = (row[i] - mean) * scale;
-    if (weight) z *= weight[i];
-    if (bias) z += bias[i];
-    if (channel_scale) z *= channel_scale[i];
-    float v = x[i] + z;
-    if (depth > 0) {
-      history[(size_t)(depth - 1) * history_stride + at + i] = v;
-      float mixed = 0.f;
-      for (int j = 0; j + 1 < depth; ++j) mixed += mix[j] * history[(size_t)j * history_stride + at + i];
-      v = mixed + mix[depth - 1] * v;
+  for (int i = threadIdx.x * V; i < width; i += step) {
+    float v[V], mixed[V];
+    if (V == 4) { const float4 a = ld4(x + i); v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w; } else v[0] = x[i];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      float z = (row[i + e] - mean) * scale;
+      if (weight) z *= weight[i + e];
+      if (bias) z += bias[i + e];
+      if (channel_scale) z *= channel_scale[i + e];
+      v[e] += z;
+      mixed[e] = 0.f;
     }
-    x[i] = v;
-    if (out) st(out + at + i, v);
+    if (depth > 0) {
+      float* mine = history + (size_t)(depth - 1) * history_stride + at + i;
+      if (V == 4) st4(mine, make_float4(v[0], v[1], v[2], v[3])); else *mine = v[0];
+#pragma unroll 4
+      for (int j = 0; j + 1 < depth; ++j) {
+        const float* theirs = history + (size_t)j * history_stride + at + i;
+        const float m = mix[j];
+        if (V == 4) {
+          const float4 a = ld4(theirs);
+          mixed[0] += m * a.x, mixed[1] += m * a.y, mixed[2] += m * a.z, mixed[3] += m * a.w;
+        } else {
+          mixed[0] += m * *theirs;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = mixed[e] + mix[depth - 1] * v[e];
+    }
+    if (V == 4) {
+      st4(x + i, make_float4(v[0], v[1], v[2], v[3]));
+      if (out) st4(out + at + i, make_float4(v[0], v[1], v[2], v[3]));
+    } else {
+      x[i] = v[0];
+      if (out) st(out + at + i, v[0]);
+    }
   }
 }
 
@@ -70,11 +105,18 @@ int qil_post_norm_scale_add(float* stream, const void* y, int y_dtype, int split
       (size_t)width * sizeof(float) > 64 * 1024)
     return -1;
   const size_t stride = (size_t)n * width, lds = (size_t)width * sizeof(float);
-  const int threads = width >= 2048 ? 512 : width >= 512 ? 256 : width >= 128 ? 128 : 64;
-#define QIL_POST_LAUNCH(TD, T, C)                                                                                      \
-  hipLaunchKernelGGL((post_norm_scale_add_kernel<TD, T, C>), dim3(n), dim3(threads), lds, s, stream, (const TD*)y, splits, \
-                     stride, weight, bias, channel_scale, eps, (T*)out, history, stride, depth, mix, width)
-#define QIL_POST_CASE(TD, T) do { if (centre) QIL_POST_LAUNCH(TD, T, 1); else QIL_POST_LAUNCH(TD, T, 0); } while (0)
+  // four neighbouring elements a thread (one 8- or 16-byte access) where the rows allow
+  const bool vec = width % 4 == 0 && (((uintptr_t)stream | (uintptr_t)y | (uintptr_t)out | (uintptr_t)history) % 16) == 0;
+  const int lanes = vec ? width / 4 : width;
+  const int threads = lanes >= 512 ? 512 : lanes >= 256 ? 256 : lanes >= 128 ? 128 : 64;
+#define QIL_POST_LAUNCH(TD, T, C, V)                                                                                   \
+  hipLaunchKernelGGL((post_norm_scale_add_kernel<TD, T, C, V>), dim3(n), dim3(threads), lds, s, stream, (const TD*)y, \
+                     splits, stride, weight, bias, channel_scale, eps, (T*)out, history, stride, depth, mix, width)
+#define QIL_POST_CASE(TD, T)                                                                                          \
+  do {                                                                                                                \
+    if (centre) { if (vec) QIL_POST_LAUNCH(TD, T, 1, 4); else QIL_POST_LAUNCH(TD, T, 1, 1); }                          \
+    else { if (vec) QIL_POST_LAUNCH(TD, T, 0, 4); else QIL_POST_LAUNCH(TD, T, 0, 1); }                                 \
+  } while (0)
   if (out_dtype == QIL_F32) {
     if (y_dtype == QIL_F32) QIL_POST_CASE(float, float); else QIL_POST_CASE(bf16_t, float);
   } else {
