@@ -282,6 +282,8 @@ def designs_phase(args, torch, dtype):
                                          num_hidden_layers=layers, num_attention_heads=z['heads'],
                                          num_key_value_heads=max(1, z['heads'] // 4), head_dim=z['dim'],
                                          max_position_embeddings=max(args.history + args.steps + args.warmup + 64, args.prefill_tokens))
+    if args.design_only:
+        models = {name: config for name, config in models.items() if args.design_only in name}
     report = {'phase': 'designs', 'design': args.design, 'sizes': args.design_sizes, 'layers': layers, 'dtype': args.dtype,
               'prefill_tokens': args.prefill_tokens, 'batch': args.batch, 'history': args.history, 'models': {}}
     for name, config in models.items():
@@ -349,6 +351,7 @@ def main():
                              'design named by --design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
     parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik', 'zinesun'], help='the design of --phase designs')
     parser.add_argument('--design-window', type=int, default=512, help='the attention window of --design zinesun')
+    parser.add_argument('--design-only', default=None, help='of the models of --phase designs, only those whose name holds this (for profiling)')
     parser.add_argument('--design-sizes', default='1b', choices=sorted(DESIGN_SIZES), help='layer sizes of --phase designs')
     parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')
     parser.add_argument('--own-products', action='store_true',

@@ -942,8 +942,14 @@ def post_norm_scale_add(stream, value, *, weight, bias, channel_scale, eps, cent
     comes back rounded to that type (what the next sub-layer's products read), else None."""
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
-    value = _plain_delta(value)
-    if isinstance(value, Partials):
+    routed = value if isinstance(value, RoutedSum) else None
+    if routed is not None:                              # the weighted sum is made as the kernel loads the row
+        top = routed.chosen.shape[1]
+        _require(routed.x, 'routed input', None, (n, width))
+        _require(routed.pairs, 'routed pairs', torch.float32, (n * top, width))
+        _require(routed.chosen, 'chosen', torch.int32, (n, top))
+        _require(routed.weights, 'weights', torch.float32, (n, top))
+    elif isinstance(value, Partials):
         _require(value.tensor, 'value', torch.float32, (value.splits, n, width))
         pointer, code, splits = value.tensor.data_ptr(), 0, value.splits
     else:
@@ -958,24 +964,28 @@ def post_norm_scale_add(stream, value, *, weight, bias, channel_scale, eps, cent
         if history.ndim != 3 or history.shape[0] < depth or tuple(history.shape[1:]) != (n, width):
             raise ValueError(f'post_norm_scale_add: history must be [>= {depth}, {n}, {width}]')
     out = torch.empty((n, width), dtype=out_dtype, device=stream.device) if out_dtype is not None else None
-    _check(library.load().qil_post_norm_scale_add(_ptr(stream), pointer, code, splits, _ptr(weight), _ptr(bias),
-                                                  _ptr(channel_scale), float(eps), int(bool(centre)), _ptr(out),
-                                                  _code(out_dtype) if out_dtype is not None else 0,
-                                                  _ptr(history) if depth else None, int(depth),
-                                                  _ptr(mix) if depth else None, n, width, _stream()), 'post_norm_scale_add')
+    tail = (_ptr(weight), _ptr(bias), _ptr(channel_scale), float(eps), int(bool(centre)), _ptr(out),
+            _code(out_dtype) if out_dtype is not None else 0, _ptr(history) if depth else None, int(depth),
+            _ptr(mix) if depth else None, n, width, _stream())
+    if routed is not None:
+        _check(library.load().qil_post_norm_scale_add_routed(_ptr(stream), _ptr(routed.pairs), _ptr(routed.weights),
+                                                             _ptr(routed.chosen), _ptr(routed.x), _code(routed.x.dtype), top,
+                                                             routed.experts, *tail), 'post_norm_scale_add_routed')
+    else:
+        _check(library.load().qil_post_norm_scale_add(_ptr(stream), pointer, code, splits, *tail), 'post_norm_scale_add')
     return out
 
 
 def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, out_dtype):
-    """x + conv(x): a causal convolution over time on every channel, conv(x)_t = sum_j weight[:, j] * x_(t - taps + 1 +
-    j), over the rows of every sequence of the step and the taps - 1 inputs before them, which are the sequence's
+    """x + conv(x): a causal convolution over time on every channel, conv(x)_t = sum_j weight[j] * x_(t - taps + 1 + j),
+    over the rows of every sequence of the step and the taps - 1 inputs before them, which are the sequence's
     state (``state`` float32 [slots, taps - 1, H]: read unless the sequence starts at position 0, and left holding
-    the sequence's last taps - 1 inputs).  ``x`` float32 [N, H] (the residual stream), ``weight`` float32 [H, taps].
-    -> [N, H] of ``out_dtype``; float32 arithmetic, one rounding."""
+    the sequence's last taps - 1 inputs).  ``x`` float32 [N, H] (the residual stream), ``weight`` float32 [taps, H]
+    (a tap's factors for all channels side by side).  -> [N, H] of ``out_dtype``; float32 arithmetic, one rounding."""
     n, width = x.shape
     _require(x, 'x', torch.float32)
-    taps = weight.shape[1]
-    _require(weight, 'weight', torch.float32, (width, taps))
+    taps = weight.shape[0]
+    _require(weight, 'weight', torch.float32, (taps, width))
     if taps > 1:
         _require(state, 'state', torch.float32)
         if state.ndim != 3 or tuple(state.shape[1:]) != (taps - 1, width):

@@ -335,6 +335,8 @@ def _declare(lib):
     lib.qil_moe_experts.restype = i
     lib.qil_post_norm_scale_add.argtypes = [p, p, i, i, p, p, p, f, i, p, i, p, i, p, i, i, p]
     lib.qil_post_norm_scale_add.restype = i
+    lib.qil_post_norm_scale_add_routed.argtypes = [p, p, p, p, p, i, i, i, p, p, p, f, i, p, i, p, i, p, i, i, p]
+    lib.qil_post_norm_scale_add_routed.restype = i
     lib.qil_short_conv.argtypes = [p, p, p, p, p, p, p, p, i, i, i, i, p]
     lib.qil_short_conv.restype = i
     lib.qil_plain_act.argtypes = [p, i, i, p, i, i, i, i, p, p]

@@ -8,7 +8,8 @@ class ShortConvolution(Part):
     [width, taps], no bias.  It reads the float32 residual stream and computes in float32; the result is rounded once
     to the type the consumer's products read.  The last taps - 1 inputs of a sequence are its state between steps:
     ``cache_need()`` is a ``StateNeed`` of [taps - 1, width] float32 (None for a single tap), and ``forward`` gets the
-    ``StateView`` of the schedule entry."""
+    ``StateView`` of the schedule entry.  ``finalize`` turns the stored weight to [taps, width], a tap's factors side
+    by side, which is how the kernel reads them."""
 
     def __init__(self, width, taps):
         super().__init__()
@@ -21,6 +22,9 @@ class ShortConvolution(Part):
 
     def cache_need(self):
         return StateNeed((self.taps - 1, self.width), 'float32') if self.taps > 1 else None
+
+    def finalize(self):
+        self.p['weight'] = self.p['weight'].t().contiguous()
 
     def forward(self, stream, ctx, cache, out_dtype):
         return ops.short_conv(stream, self.p['weight'], state=cache.state if cache is not None else None,

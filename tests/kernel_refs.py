@@ -223,7 +223,7 @@ def post_norm_scale_add(stream, value, *, weight, bias, channel_scale, eps, cent
 
 
 def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, out_dtype):
-    taps, keep = weight.shape[1], weight.shape[1] - 1
+    taps, keep = weight.shape[0], weight.shape[0] - 1               # weight [taps, H]
     out = torch.empty_like(x)
     for s in range(n_seqs):
         first, last, start = int(cu_seqlens[s]), int(cu_seqlens[s + 1]), int(seq_starts[s])
@@ -233,7 +233,7 @@ def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, 
             before[:max(0, keep - start)] = 0.0                 # places before the sequence's start
         inputs = torch.cat([before, x[first:last]])
         for t in range(last - first):
-            out[first + t] = x[first + t] + (weight.t() * inputs[t:t + taps]).sum(dim=0)
+            out[first + t] = x[first + t] + (weight * inputs[t:t + taps]).sum(dim=0)
         if keep:
             state[int(seq_slots[s])] = inputs[-keep:]
     return out.to(out_dtype)

@@ -26,20 +26,21 @@ def ints(values):
 # ------------------------------------------------------------------------------------------------ short convolution
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('width', [20, 21, 7, 1028, 1300])
-@pytest.mark.parametrize('taps', [1, 2, 3, 4])
+@pytest.mark.parametrize('taps', [1, 2, 3, 4, 6])
 def test_short_convolution_with_its_state(dtype, width, taps):
-    """Three steps over five slots: sequences that begin (whatever their slot held before, NaN here, is not read), that
+    """Five steps over five slots: sequences that begin (whatever their slot held before, NaN here, is not read), that
     continue from a state shorter than taps - 1 inputs, that bring fewer rows than the state holds, and one long
     portion; a slot is given to a new sequence in the last step."""
     g = torch.Generator().manual_seed(width * 10 + taps)
     keep = taps - 1
-    weight = torch.randn(width, taps, generator=g)
+    weight = torch.randn(taps, width, generator=g)
     state_c = torch.full((5, keep, width), float('nan')) if keep else None
     state_g = state_c.clone().cuda() if keep else None
     steps = [([5, 1, 2], [0, 0, 0], [3, 0, 4]),                  # (rows, positions before the step, slots)
              ([1, 1, 70], [5, 1, 2], [3, 0, 4]),
              ([2, 1, 3, 1], [6, 2, 0, 72], [3, 0, 1, 4]),
-             ([9, 2], [0, 8], [0, 3])]                           # slot 0 begins anew
+             ([9, 2], [0, 8], [0, 3]),                           # slot 0 begins anew
+             ([1100, 1, 2, 9, 30], [10, 9, 0, 0, 0], [3, 0, 1, 2, 4])]       # enough rows for threads that walk several
     for counts, starts, slots in steps:
         n = sum(counts)
         x = torch.randn(n, width, generator=g)
@@ -63,8 +64,8 @@ def test_each_tap_reads_the_input_that_many_steps_back():
     nothing before the sequence's start, through steps of any size."""
     width, taps = 8, 4
     for tap in range(taps):
-        weight = torch.zeros(width, taps)
-        weight[:, tap] = 1.0
+        weight = torch.zeros(taps, width)
+        weight[tap] = 1.0
         back = taps - 1 - tap
         state = torch.full((2, taps - 1, width), float('nan')).cuda()
         inputs = torch.arange(1, 21, dtype=torch.float32)[:, None].repeat(1, width)
@@ -144,6 +145,43 @@ def test_a_normed_output_joins_the_stream_with_a_channel_scale_and_an_average_ov
                                    eps=1e-5, centre=centre) is None
     y = value.float() - (value.float().mean(-1, keepdim=True) if centre else 0.0)
     close(s_gpu, stream + y / torch.sqrt(y.square().mean(-1, keepdim=True) + 1e-5) * weight + bias, torch.float32, 10.0)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('width', [40, 37, 1100])
+def test_a_routed_sum_is_made_as_the_row_is_loaded(dtype, width):
+    """A routed feed-forward's pairs in the place of the value: the weighted sum in slot order, an identity expert's
+    pair being the token's own input; as the sum's own kernel followed by the plain form."""
+    g = torch.Generator().manual_seed(width)
+    n, top, experts = 7, 3, 5
+    stream = torch.randn(n, width, generator=g)
+    x = torch.randn(n, width, generator=g).to(dtype)
+    pairs = torch.randn(n * top, width, generator=g) * 2
+    chosen = torch.randint(0, experts + 2, (n, top), generator=g).to(torch.int32)       # two identity experts behind the five
+    chosen[0] = torch.tensor([experts, 0, experts + 1])
+    weights = torch.rand(n, top, generator=g)
+    weight, bias, channel = (torch.randn(width, generator=g) for _ in range(3))
+    history, mix = torch.randn(3, n, width, generator=g), torch.randn(3, generator=g)
+    picked = torch.where((chosen >= experts)[:, :, None], x.float()[:, None, :].expand(n, top, width), pairs.view(n, top, width))
+    summed = (weights[:, :, None] * picked).sum(dim=1)
+    for depth in (0, 3):
+        routed = ops.RoutedSum(x.cuda(), pairs.cuda(), chosen.cuda(), weights.cuda(), experts)
+        s_gpu, s_two, s_cpu = stream.clone().cuda(), stream.clone().cuda(), stream.clone()
+        h_gpu, h_two, h_cpu = history.clone().cuda(), history.clone().cuda(), history.clone()
+        args = dict(weight=weight, bias=bias, channel_scale=channel)
+        rest = dict(eps=1e-5, centre=True, out_dtype=dtype, depth=depth)
+        on_gpu = {k: v.cuda() for k, v in args.items()}
+        got = ops.post_norm_scale_add(s_gpu, routed, history=h_gpu if depth else None, mix=mix.cuda() if depth else None,
+                                      **on_gpu, **rest)
+        two = ops.post_norm_scale_add(s_two, ops.Partials(routed.materialize().unsqueeze(0)), history=h_two if depth else None,
+                                      mix=mix.cuda() if depth else None, **on_gpu, **rest)
+        want = refs.post_norm_scale_add(s_cpu, summed, history=h_cpu if depth else None, mix=mix if depth else None, **args, **rest)
+        close(got, want, dtype, 10.0)
+        close(s_gpu, s_cpu, torch.float32, 10.0)
+        close(h_gpu, h_cpu, torch.float32, 10.0)
+        close(got, two.cpu(), dtype)
+        close(s_gpu, s_two.cpu(), torch.float32)
+        close(h_gpu, h_two.cpu(), torch.float32)
 
 
 # ------------------------------------------------------------------------------------------------ window and gate
