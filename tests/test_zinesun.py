@@ -60,8 +60,24 @@ def _narrow():
     return plain.make_config(layers, vocab=50, width=20, taps=2, scale=2.0)
 
 
-# (configuration, seed, page size, spread of the matrices)
-CONFIGS = {'mixed': (_mixed(), 11, 8, 1.0), 'wide': (_wide(), 12, 16, 0.8), 'narrow': (_narrow(), 13, 4, 1.2)}
+def _odd():
+    # sizes that are multiples of nothing (a width the four-wide kernels do not take), five taps (more than the
+    # convolution keeps in registers), a first layer without a feed-forward, every expert chosen and one of many
+    layers = [
+        plain.layer(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=36, q_rank=22, scale=0.3, window=7),
+        plain.layer(heads=2, dim=6, rot_dim=2, vdim=6, kv_rank=10, q_rank=10, scale=0.5, window=19, base=77.0,
+                    mlp=plain.moe_mlp(ff=10, experts=4, top=4)),
+        plain.layer(heads=5, dim=4, rot_dim=4, vdim=2, kv_rank=18, q_rank=6, scale=0.45, window=3, mlp=plain.dense_mlp(50)),
+        plain.layer(heads=1, dim=2, rot_dim=10, vdim=30, kv_rank=6, q_rank=2, scale=0.6, window=40, base=5.0,
+                    mlp=plain.moe_mlp(ff=7, experts=9, top=1)),
+    ]
+    return plain.make_config(layers, vocab=101, width=30, taps=5, scale=1.7, eps=1e-4)
+
+
+# (configuration, seed, page size, spread of the matrices); 'odd' runs on the GPU only (the others cover the host code)
+CONFIGS = {'mixed': (_mixed(), 11, 8, 1.0), 'wide': (_wide(), 12, 16, 0.8), 'narrow': (_narrow(), 13, 4, 1.2),
+           'odd': (_odd(), 14, 8, 1.0)}
+GPU_ONLY = {'odd'}
 
 
 def tokens_for(config, length, seed):
@@ -153,6 +169,8 @@ def make_case(name, config, weights, backend, folder, page_size):
 
 @pytest.fixture(params=sorted(CONFIGS))
 def case(request, backend, tmp_path):
+    if request.param in GPU_ONLY and backend[0] == 'cpu':
+        pytest.skip('this configuration runs on the GPU only')
     config, seed, page_size, spread = CONFIGS[request.param]
     return make_case(request.param, config, plain.random_weights(config, seed, spread), backend, tmp_path / request.param, page_size)
 
