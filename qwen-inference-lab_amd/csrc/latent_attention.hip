@@ -92,17 +92,18 @@ __global__ void head_product_kernel(const TX* __restrict__ x, int x_row, int x_h
 }
 
 // The same product for few rows (decoding): the weights of a head are then read by too few blocks for the chip, so a
-// block takes 8 rows, 64 outputs and splits k 32 ways: a thread reads 8 consecutive outputs of every 32nd k (16 bytes
-// of bfloat16), and the 32 partial sums meet by shuffles in a wave and through LDS between the four waves.
-// Takes o_dim % 8 == 0 and w aligned to 8 elements.
-template <typename TX, typename TW, typename TO>
+// block takes 8 rows, OT * 8 outputs (OT = 8, or 4 where that still leaves few blocks) and splits k 256 / OT ways: a
+// thread reads 8 consecutive outputs of every (256 / OT)th k (16 bytes of bfloat16), and the partial sums meet by
+// shuffles in a wave and through LDS between the four waves.  Takes o_dim % 8 == 0 and w aligned to 8 elements.
+template <typename TX, typename TW, typename TO, int OT>
 __global__ void __launch_bounds__(256)
 head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const TW* __restrict__ w, TO* __restrict__ out,
                         int out_row, int out_head, int n_rows, int k_dim, int o_dim) {
-  extern __shared__ float xs[];                       // [8][k_dim], then [4 waves][8 rows][64 outputs]
+  constexpr int OB = OT * 8, KG = 256 / OT;           // outputs a block, k groups
+  extern __shared__ float xs[];                       // [8][k_dim], then [4 waves][8 rows][OB outputs]
   float* sums = xs + 8 * k_dim;
-  const int row0 = blockIdx.x * 8, h = blockIdx.y, tid = threadIdx.x, to = tid & 7, kg = tid >> 3;
-  const int o0 = blockIdx.z * 64 + to * 8;
+  const int row0 = blockIdx.x * 8, h = blockIdx.y, tid = threadIdx.x, to = tid % OT, kg = tid / OT;
+  const int o0 = blockIdx.z * OB + to * 8;
 #pragma unroll 4
   for (int idx = tid; idx < 8 * k_dim; idx += 256) {
     const int r = idx / k_dim, k = idx - r * k_dim;
@@ -113,7 +114,7 @@ head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const T
   if (o0 < o_dim) {
     const TW* wh = w + (size_t)h * k_dim * o_dim + o0;
 #pragma unroll 4                                      // four weight reads on their way at a time
-    for (int k = kg; k < k_dim; k += 32) {
+    for (int k = kg; k < k_dim; k += KG) {
       float wv[8];
       ld8(wh + (size_t)k * o_dim, wv);
 #pragma unroll
@@ -129,24 +130,23 @@ head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const T
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float v = acc[r][j];
-      v += __shfl_xor(v, 8, QIL_WAVE);
-      v += __shfl_xor(v, 16, QIL_WAVE);
-      v += __shfl_xor(v, 32, QIL_WAVE);
+#pragma unroll
+      for (int step = OT; step < QIL_WAVE; step *= 2) v += __shfl_xor(v, step, QIL_WAVE);
       acc[r][j] = v;
     }
   const int wave = tid >> 6;
-  if ((tid & 63) < 8) {
+  if ((tid & 63) < OT) {
 #pragma unroll
     for (int r = 0; r < 8; ++r)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) sums[(wave * 8 + r) * 64 + to * 8 + j] = acc[r][j];
+      for (int j = 0; j < 8; ++j) sums[(wave * 8 + r) * OB + to * 8 + j] = acc[r][j];
   }
   __syncthreads();
-  for (int idx = tid; idx < 8 * 64; idx += 256) {
-    const int r = idx / 64, j = idx % 64, o = blockIdx.z * 64 + j;
+  for (int idx = tid; idx < 8 * OB; idx += 256) {
+    const int r = idx / OB, j = idx % OB, o = blockIdx.z * OB + j;
     if (row0 + r < n_rows && o < o_dim)
       st(out + (size_t)(row0 + r) * out_row + (size_t)h * out_head + o,
-         sums[r * 64 + j] + sums[(8 + r) * 64 + j] + sums[(16 + r) * 64 + j] + sums[(24 + r) * 64 + j]);
+         sums[r * OB + j] + sums[(8 + r) * OB + j] + sums[(16 + r) * OB + j] + sums[(24 + r) * OB + j]);
   }
 }
 
@@ -292,8 +292,11 @@ int qil_latent_prepare(const void* x, int x_dtype, int splits, const float* wq, 
   const size_t stride = (size_t)n * (q_rank + rank + rot + gates);
   const size_t row_bytes = (size_t)(q_rank + rank + rot + gates) * sizeof(float);
   const int held = row_bytes <= 48 * 1024;            // the row's sums fit in LDS
+  // a thread's loads of the row come one after the other: with few rows (too few blocks to hide that) wide rows get
+  // more threads, not more turns
+  const int total = q_rank + rank + rot + gates, threads = n > 64 ? 256 : total >= 2048 ? 1024 : total >= 1024 ? 512 : 256;
 #define QIL_LP(TD, T)                                                                                               \
-  hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(256), held ? row_bytes : 0, s, (const TD*)x, splits, \
+  hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(threads), held ? row_bytes : 0, s, (const TD*)x, splits, \
                      stride, wq, wc, freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, gate_out, q_rank, rank, rot, gates, eps, held)
   if (dtype == QIL_F32) {
     if (x_dtype != QIL_F32) return -1;
@@ -321,10 +324,15 @@ int qil_head_product(const void* x, int x_dtype, int x_row, int x_head, const vo
   const size_t w_bytes = w_dtype == QIL_F32 ? 4 : 2;
   const bool few = n <= 32 && o_dim % 8 == 0 && (size_t)w % (8 * w_bytes) == 0 && lds + 4 * 8 * 64 * sizeof(float) <= 64 * 1024;
   const dim3 grid_few((n + 7) / 8, heads, (o_dim + 63) / 64);
+  const bool narrow = grid_few.x * grid_few.y * grid_few.z < 128;      // few blocks: 32 outputs a block, k split 64 ways
+  const dim3 grid_narrow((n + 7) / 8, heads, (o_dim + 31) / 32);
 #define QIL_HP(TX, TW, TO)                                                                                            \
   do {                                                                                                                  \
-    if (few)                                                                                                            \
-      hipLaunchKernelGGL((head_product_few_kernel<TX, TW, TO>), grid_few, dim3(256), lds + 4 * 8 * 64 * sizeof(float), s, \
+    if (few && narrow)                                                                                                  \
+      hipLaunchKernelGGL((head_product_few_kernel<TX, TW, TO, 4>), grid_narrow, dim3(256), lds + 4 * 8 * 32 * sizeof(float), s, \
+                         (const TX*)x, x_row, x_head, (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim);       \
+    else if (few)                                                                                                       \
+      hipLaunchKernelGGL((head_product_few_kernel<TX, TW, TO, 8>), grid_few, dim3(256), lds + 4 * 8 * 64 * sizeof(float), s, \
                          (const TX*)x, x_row, x_head, (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim);       \
     else                                                                                                                \
       hipLaunchKernelGGL((head_product_kernel<TX, TW, TO, 8>), grid, dim3(threads), lds, s, (const TX*)x, x_row, x_head, \
