@@ -557,3 +557,34 @@ def test_trace_replay_program(tmp_path, dtype):
             if (expected[request].margin[:max(places) + 1] < NEAR_TIE[judge.dtype]).any():
                 continue                                       # a close call of a router somewhere before: rounding's to make
             judge.close(got, expected[request][places], f'{shape} {request}')
+
+
+@pytest.mark.gpu
+def test_command_line(tmp_path):
+    """``python -m qil_amd`` on a Zinesun folder: greedy generation through the scheduler in portions of two tokens
+    equals the plain model's, and a folder written from a configuration with a seed generates with a temperature."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    config, seed, _, spread = CONFIGS['narrow']
+    weights = plain.random_weights(config, seed, spread)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    prompt, out = [5, 17, 3, 41, 8, 8, 30], tmp_path / 'result.json'
+    run = subprocess.run([sys.executable, '-m', 'qil_amd', '--model', str(folder), '--token-ids', json.dumps(prompt),
+                          '--dtype', 'float32', '--max-new-tokens', '6', '--pages', '8', '--page-size', '4',
+                          '--chunk-size', '2', '--ignore-eos', '--output', str(out)],
+                         cwd=root, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    result = json.loads(out.read_text())
+    assert result['token_ids'] == plain.greedy(prompt, 6, weights, config) and result['state'] == 'completed'
+    elsewhere = tmp_path / 'elsewhere'
+    elsewhere.mkdir()
+    run = subprocess.run([sys.executable, '-m', 'qil_amd', '--model', str(tmp_path / 'random'), '--random-config',
+                          json.dumps(CONFIGS['mixed'][0]), '--random-seed', '3', '--token-ids', '[1, 2, 3]', '--dtype',
+                          'bfloat16', '--max-new-tokens', '4', '--temperature', '0.7', '--seed', '5', '--ignore-eos'],
+                         cwd=elsewhere, env=dict(os.environ, PYTHONPATH=str(root)), capture_output=True, text=True,
+                         timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert len(json.loads(run.stdout[run.stdout.index('{'):])['token_ids']) == 4
