@@ -232,8 +232,8 @@ def short_conv(x, weight, *, state, cu_seqlens, seq_starts, seq_slots, row_seq, 
             before = state[int(seq_slots[s])].clone()
             before[:max(0, keep - start)] = 0.0                 # places before the sequence's start
         inputs = torch.cat([before, x[first:last]])
-        for t in range(last - first):
-            out[first + t] = x[first + t] + (weight * inputs[t:t + taps]).sum(dim=0)
+        rows = last - first
+        out[first:last] = x[first:last] + sum(weight[j] * inputs[j:j + rows] for j in range(taps))
         if keep:
             state[int(seq_slots[s])] = inputs[-keep:]
     return out.to(out_dtype)

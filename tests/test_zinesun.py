@@ -74,10 +74,11 @@ def _odd():
     return plain.make_config(layers, vocab=101, width=30, taps=5, scale=1.7, eps=1e-4)
 
 
-# (configuration, seed, page size, spread of the matrices); 'odd' runs on the GPU only (the others cover the host code)
+# (configuration, seed, page size, spread of the matrices); 'wide' (made for the matrix-core kernel) and 'odd' run on
+# the GPU only: the plain references are slow, and the other two cover the host code
 CONFIGS = {'mixed': (_mixed(), 11, 8, 1.0), 'wide': (_wide(), 12, 16, 0.8), 'narrow': (_narrow(), 13, 4, 1.2),
            'odd': (_odd(), 14, 8, 1.0)}
-GPU_ONLY = {'odd'}
+GPU_ONLY = {'odd', 'wide'}
 
 
 def tokens_for(config, length, seed):
