@@ -4,5 +4,6 @@ from .qwen3 import Qwen3Config
 from .fubapel import FubapelConfig
 from .gerivik import GerivikConfig
 from .zinesun import ZinesunConfig
+from .dogozen import DogozenConfig
 
-__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig', 'GerivikConfig', 'ZinesunConfig']
+__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig', 'GerivikConfig', 'ZinesunConfig', 'DogozenConfig']

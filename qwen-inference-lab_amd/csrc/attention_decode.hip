@@ -67,7 +67,8 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
                    const int* __restrict__ row_seq, const int* __restrict__ positions,
                    const int* __restrict__ row_index, float* __restrict__ part_acc, float* __restrict__ part_m,
                    float* __restrict__ part_l, bf16_t* __restrict__ out, int heads, int kv_heads, int d,
-                   int page_size, int window, float scale, int P, int parts, float softcap) {
+                   int page_size, int window, float scale, int P, int parts, float softcap,
+                   const float* __restrict__ sinks) {
   constexpr int QFRAGS = DMAX / 32, DTILES = DMAX / 16;
   if (WHOLE) d = DMAX;                                      // what the host has checked, known to the compiler: no
                                                             // condition on the head size stays in the loops
@@ -343,7 +344,8 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
     }
     const int head = kvh * g + h;
     if (parts == 1) {
-      out[((size_t)row * heads + head) * d + e] = f32_to_bf16(total / ll);
+      out[((size_t)row * heads + head) * d + e] =
+          f32_to_bf16(sinks ? total * sink_reciprocal(ll, mm, sinks[head]) : total / ll);
     } else {
       const size_t c = ((size_t)slot_row * heads + head) * parts + part;
       part_acc[c * d + e] = total;
@@ -362,12 +364,13 @@ extern "C" int qil_attn_decode_takes(int heads, int kv_heads, int d, int page_si
 // Partial results in the layout of the row kernel (acc [rows, heads, parts, d], then m, then l);
 // the caller runs the row kernel's merge when parts > 1.  P must be a multiple of 32; a block has
 // `waves` waves (at most 8), best one or two 32-key steps of P for each.  pairs != 0: a wave loads two of
-// its steps at a time (twice the registers; for launches of at most one block a CU).
+// its steps at a time (twice the registers; for launches of at most one block a CU).  sinks: null, or float32 [heads]:
+// exp(sink) joins a head's divisor (here when parts == 1, else in the merge).
 extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* block_tables, int table_stride, const int* row_seq, const int* positions,
                                const int* row_index, void* workspace, void* out, int rows, int heads, int kv_heads,
                                int d, int page_size, int window, float scale, int P, int parts, int waves,
-                               int pairs, float softcap, hipStream_t s) {
+                               int pairs, float softcap, const float* sinks, hipStream_t s) {
   if (rows == 0) return 0;
   if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || P % 32 || P < 32 || parts < 1 || parts > 65535 ||
       kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES)
@@ -383,12 +386,12 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
   hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, FUSED>), grid, dim3(waves * QIL_WAVE), lds, s, FIELDS,         \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                      table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
-                     page_size, window, scale, P, parts, softcap)
+                     page_size, window, scale, P, parts, softcap, sinks)
 #define QIL_DEC_WHOLE(DMAX, PAIRS)                                                                                  \
   hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, false, true>), grid, dim3(waves * QIL_WAVE), lds, s, none,     \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                      table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
-                     page_size, window, scale, P, parts, softcap)
+                     page_size, window, scale, P, parts, softcap, sinks)
 #define QIL_DEC_CASE(DMAX)                                                                                          \
   if (d == DMAX && pairs) QIL_DEC_WHOLE(DMAX, true);                                                                \
   else if (d == DMAX) QIL_DEC_WHOLE(DMAX, false);                                                                   \
@@ -447,6 +450,7 @@ extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* 
   const void* q = nullptr;
   const int q_stride = 0;
   const int* row_index = nullptr;
+  const float* sinks = nullptr;
 #define QIL_DEC_CASE(DMAX)                                                                                          \
   if (pairs) QIL_DEC_LAUNCH(DMAX, true, true, fused);                                                               \
   else QIL_DEC_LAUNCH(DMAX, false, true, fused)

@@ -54,7 +54,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
                          const int* __restrict__ row_index, float* __restrict__ part_acc,
                          float* __restrict__ part_m, float* __restrict__ part_l,
                          T* __restrict__ out, int heads, int kv_heads, int d, int page_size, int window,
-                         float scale, float softcap, int P, int parts, int tg_log2) {
+                         float scale, float softcap, int P, int parts, int tg_log2, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;   // slot_row indexes the workspace
   const int row = row_index ? row_index[slot_row] : slot_row;             // row of the step's batch
@@ -215,7 +215,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
       for (int hh = 0; hh < GT; ++hh)
         if (hh == h) { m = m_h[hh]; l = l_h[hh]; }
       if (parts == 1) {
-        st(out + ((size_t)row * heads + head) * d + e, total / l);
+        st(out + ((size_t)row * heads + head) * d + e, sinks ? total * sink_reciprocal(l, m, sinks[head]) : total / l);
       } else {
         const size_t cell = ((size_t)slot_row * heads + head) * parts + part;
         part_acc[cell * d + e] = total;
@@ -233,7 +233,7 @@ __global__ void __launch_bounds__(QIL_WAVE)
 attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
                        const float* __restrict__ part_l, const int* __restrict__ positions,
                        const int* __restrict__ row_index, T* __restrict__ out, int heads, int d,
-                       int window, int P, int parts, int tg) {
+                       int window, int P, int parts, int tg, const float* __restrict__ sinks) {
   const int slot_row = blockIdx.x;
   const int head = blockIdx.y * (QIL_WAVE / tg) + threadIdx.x / tg, e = (threadIdx.x % tg) * 4;
   const bool head_there = head < heads;                    // the same for the tg lanes of a head; all of them take part in the maximum
@@ -275,6 +275,11 @@ attn_rows_merge_kernel(const float* __restrict__ part_acc, const float* __restri
     }
   }
   T* to = out + ((size_t)row * heads + head) * d + e;
+  if (sinks) {                                             // the sink joins the divisor once, here
+    const float r = sink_reciprocal(denom, m, sinks[head]);
+    st(to, numer.x * r); st(to + 1, numer.y * r); st(to + 2, numer.z * r); st(to + 3, numer.w * r);
+    return;
+  }
   st(to, numer.x / denom); st(to + 1, numer.y / denom); st(to + 2, numer.z / denom); st(to + 3, numer.w / denom);
 }
 
@@ -300,7 +305,8 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
                        int table_stride, const int* row_seq, const int* positions, const int* row_index,
                        float* part_acc, float* part_m,
                        float* part_l, void* out, int rows, int heads, int kv_heads, int d, int page_size, int window,
-                       float scale, float softcap, int P, int parts, hipStream_t s, bool merge = true) {
+                       float scale, float softcap, int P, int parts, hipStream_t s, bool merge = true,
+                       const float* sinks = nullptr) {
   const int g = heads / kv_heads;
   const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;            // head tile: 1, 2, 4 or 8
   const int tg_log2 = next_pow2_log2((d + 7) / 8);
@@ -310,7 +316,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
   hipLaunchKernelGGL((attn_rows_partial_kernel<T, GT>), grid, dim3(ATT_THREADS), lds, s, (const T*)q, q_stride,    \
                      (const T*)k_cache, (const T*)v_cache, block_tables, table_stride, row_seq, positions,         \
                      row_index, part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, softcap, P, parts,    \
-                     tg_log2)
+                     tg_log2, sinks)
   switch (gt) {
     case 1: QIL_ROWS_CASE(1); break;
     case 2: QIL_ROWS_CASE(2); break;
@@ -324,7 +330,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
   dim3 merge_grid;
   merge_shape(rows, heads, d, &tg, &merge_grid);
   hipLaunchKernelGGL(attn_rows_merge_kernel<T>, merge_grid, dim3(QIL_WAVE), 0, s, part_acc, part_m, part_l, positions,
-                     row_index, (T*)out, heads, d, window, P, parts, tg);
+                     row_index, (T*)out, heads, d, window, P, parts, tg, sinks);
   return (int)hipGetLastError();
 }
 
@@ -338,12 +344,13 @@ size_t qil_attn_rows_workspace(int rows, int heads, int d, int parts) {
 // q: rows of stride q_stride elements, head h at offset h * d.  out: [all rows, heads * d].
 // row_index: null (the kernel's rows are the batch's rows 0 .. rows-1) or the batch rows to serve.
 // workspace: qil_attn_rows_workspace bytes.  P: keys per part, parts = ceil(max context / P).
+// sinks: null, or float32 [heads] (a term exp(sink) more in every head's divisor).
 // Requires d % 8 == 0, d <= 256, P <= 1024.  Returns -1 on a size it does not take.
 int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                   int table_stride, const int* row_seq, const int* positions, const int* row_index, void* workspace,
                   void* out, int rows,
                   int heads, int kv_heads, int d, int page_size, int window, float scale, float softcap, int P, int parts, int dtype,
-                  hipStream_t s) {
+                  const float* sinks, hipStream_t s) {
   if (rows == 0) return 0;
   if (d % 8 || d > 256 || d < 8 || heads % kv_heads || P < 1 || P > 1024 || parts < 1 || parts > 65535 ||
       kv_heads > 65535) return -1;
@@ -355,9 +362,9 @@ int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* 
   float* l = m ? m + (size_t)rows * heads * parts : nullptr;
   if (dtype == QIL_F32)
     return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
-                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s);
+                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s, true, sinks);
   return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
-                             acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s);
+                             acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s, true, sinks);
 }
 
 // The same without the merge: the parts' results stay in the workspace for a consumer that merges them itself
@@ -383,8 +390,9 @@ int qil_attn_rows_unmerged(const void* q, int q_stride, const void* k_cache, con
 }
 
 // Merge of partial results written by a partial kernel (this file's or the matrix-core decode kernel's).
+// sinks: null, or float32 [heads]: exp(sink) joins every head's divisor once.
 int qil_attn_merge(const void* workspace, const int* positions, const int* row_index, void* out, int rows, int heads,
-                   int d, int window, int P, int parts, int dtype, hipStream_t s) {
+                   int d, int window, int P, int parts, int dtype, const float* sinks, hipStream_t s) {
   if (rows == 0 || parts <= 1) return 0;
   const float* acc = (const float*)workspace;
   const float* m = acc + (size_t)rows * heads * parts * d;
@@ -396,10 +404,10 @@ int qil_attn_merge(const void* workspace, const int* positions, const int* row_i
   const dim3 block(QIL_WAVE);
   if (dtype == QIL_F32)
     hipLaunchKernelGGL(attn_rows_merge_kernel<float>, grid, block, 0, s, acc, m, l, positions, row_index, (float*)out,
-                       heads, d, window, P, parts, tg);
+                       heads, d, window, P, parts, tg, sinks);
   else
     hipLaunchKernelGGL(attn_rows_merge_kernel<bf16_t>, grid, block, 0, s, acc, m, l, positions, row_index, (bf16_t*)out,
-                       heads, d, window, P, parts, tg);
+                       heads, d, window, P, parts, tg, sinks);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -64,7 +64,7 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
                  int page_size, int window, float scale, int GH, int chunks, int ps_shift,
                  float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P, int parts,
-                 float softcap) {
+                 float softcap, const float* __restrict__ sinks) {
   // with a soft cap the scores are scaled and capped as they are made, and nothing is left for the exponent to scale
   const float raw_scale = scale;
   if (softcap > 0.f) scale = 1.f;
@@ -472,6 +472,17 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
     }
     // a division, as in the merge of parts: keys that all lie in one part then give the same bits either way
     T* orow = out + ((size_t)(q0 + my_row[b]) * heads + head) * d;
+    if (sinks) {                                            // one more term in the divisor: exp(sink), no key, no value
+      const float r = sink_reciprocal(total, m[b] * scale, sinks[head]);
+#pragma unroll
+      for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int dim = t * 16 + 4 * kb + i;
+          if (WHOLE || dim < d) st(orow + dim, o[b][t][i] * r);
+        }
+      continue;
+    }
 #pragma unroll
     for (int t = 0; t < DTILES; ++t)
 #pragma unroll
@@ -487,7 +498,7 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                        int max_query, int heads, int kv_heads, int d, int page_size, int window, float scale,
                        hipStream_t s, float* workspace = nullptr, int total_rows = 0, int P = 0, int parts = 1,
-                       float softcap = 0.f) {
+                       float softcap = 0.f, const float* sinks = nullptr) {
   using TT = TileTraits<T>;
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
@@ -511,7 +522,7 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
     if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(TILE_THREADS), lds, s, (const T*)q, q_stride, (const T*)k_cache,
                      (const T*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (T*)out, heads, kv_heads, d,
-                     page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts, softcap);
+                     page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts, softcap, sinks);
   return (int)hipGetLastError();
 }
 
@@ -561,20 +572,20 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
                          const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
                          void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
                          int window, float scale, int dtype, hipStream_t s, float* workspace, int total_rows, int P,
-                         int parts, float softcap) {
+                         int parts, float softcap, const float* sinks = nullptr) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
   // capped scores of bfloat16 heads of 128: the prompt kernel's capped form (keys in one part or in parts of whole tiles)
-  if (softcap > 0.f && dtype == QIL_BF16 && qil_attn_prompt_takes(d, page_size, table_stride) && (parts == 1 || P % 64 == 0))
+  if (softcap > 0.f && !sinks && dtype == QIL_BF16 && qil_attn_prompt_takes(d, page_size, table_stride) && (parts == 1 || P % 64 == 0))
     return qil_attn_prompt_capped(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                   n_seqs, max_query, heads, kv_heads, page_size, window, scale, softcap, workspace,
                                   total_rows, P, parts, s);
-  if (parts == 1 && softcap <= 0.f && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
+  if (parts == 1 && softcap <= 0.f && !sinks && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
     return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);
 #define QIL_TILE_CASE(T, DMAX)                                                                                      \
   return launch_tile<T, DMAX, (sizeof(T) == 2 && DMAX <= 128) ? 2 : 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
-                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s, workspace, total_rows, P, parts, softcap)
+                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s, workspace, total_rows, P, parts, softcap, sinks)
   if (dtype == QIL_F32) {
     if (d <= 64) QIL_TILE_CASE(float, 64);
     if (d <= 128) QIL_TILE_CASE(float, 128);
@@ -589,9 +600,9 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
 extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                              const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
                              void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
-                             int window, float scale, float softcap, int dtype, hipStream_t s) {
+                             int window, float scale, float softcap, int dtype, const float* sinks, hipStream_t s) {
   return tile_dispatch(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
-                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, nullptr, 0, 0, 1, softcap);
+                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, nullptr, 0, 0, 1, softcap, sinks);
 }
 
 extern "C" int qil_attn_tile_in_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,

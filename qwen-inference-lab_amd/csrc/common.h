@@ -47,6 +47,15 @@ __device__ __forceinline__ float soft_cap_fast(float score, float cap, float dou
   return cap - 2.f * cap * __builtin_amdgcn_rcpf(t + 1.f);                       // cap * (1 - 2 / (t + 1))
 }
 
+// A sink in a softmax: one more term exp(sink) in the denominator, with no key and no value.  With the sum l of
+// exp(score - m) over the keys, the weights' divisor is l + exp(sink - m); this is its reciprocal, made so that a
+// sink far above every score does not overflow.
+__device__ __forceinline__ float sink_reciprocal(float l, float m, float sink) {
+  if (sink <= m) return 1.f / (l + expf(sink - m));
+  const float t = expf(m - sink);
+  return t / (l * t + 1.f);
+}
+
 // Value after a round trip through T (what the reference's cast to the model dtype does).
 template <typename T> __device__ __forceinline__ float round_to(float v);
 template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }

@@ -86,7 +86,8 @@ moe_logits_kernel(const T* __restrict__ x, int n, int width, const float* __rest
 __global__ void __launch_bounds__(MOE_ROUTE_THREADS)
 moe_select_kernel(const float* __restrict__ logits, int n, const float* __restrict__ bias,
                   const float* __restrict__ correction, int outputs, int groups,
-                  int keep, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weights) {
+                  int keep, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weights,
+                  int sigmoid_scores, int group_top2, float weight_scale, float renormalize_eps) {
   extern __shared__ float lds[];                        // per wave: [outputs] scores, [outputs] choice scores, [groups]
   const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
   float* score = lds + (size_t)wave * (2 * outputs + groups);
@@ -96,24 +97,36 @@ moe_select_kernel(const float* __restrict__ logits, int n, const float* __restri
   const bool live = n_row < n;
   const float* z = logits + (size_t)min(n_row, n - 1) * outputs;
   auto logit = [&](int e) { return z[e] + (bias ? bias[e] : 0.f); };
-  float top_logit = -INFINITY;
-  for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, logit(e));
-  top_logit = wave_max(top_logit);
-  float total = 0.f;
-  for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(logit(e) - top_logit);
-  total = wave_sum(total);
-  for (int e = lane; e < outputs; e += QIL_WAVE) {
-    const float s = expf(logit(e) - top_logit) / total;
-    score[e] = s;
-    choice[e] = correction ? s + correction[e] : logit(e);
+  if (sigmoid_scores) {                                 // every output by itself; the choice goes by the score
+    for (int e = lane; e < outputs; e += QIL_WAVE) {
+      const float s = 1.f / (1.f + expf(-logit(e)));
+      score[e] = s;
+      choice[e] = correction ? s + correction[e] : s;
+    }
+  } else {
+    float top_logit = -INFINITY;
+    for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, logit(e));
+    top_logit = wave_max(top_logit);
+    float total = 0.f;
+    for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(logit(e) - top_logit);
+    total = wave_sum(total);
+    for (int e = lane; e < outputs; e += QIL_WAVE) {
+      const float s = expf(logit(e) - top_logit) / total;
+      score[e] = s;
+      choice[e] = correction ? s + correction[e] : logit(e);
+    }
   }
   __syncthreads();
   if (groups > 1 && keep < groups) {
     const int size = outputs / groups;
     for (int g = lane; g < groups; g += QIL_WAVE) {
-      float best = -INFINITY;
-      for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, choice[e]);
-      group_best[g] = best;
+      float best = -INFINITY, second = -INFINITY;
+      for (int e = g * size; e < (g + 1) * size; ++e) {
+        const float v = choice[e];
+        if (v > best) { second = best; best = v; }
+        else if (v > second) second = v;
+      }
+      group_best[g] = group_top2 && size > 1 ? best + second : best;     // its largest, or the sum of its two largest
     }
     __syncthreads();
     // the `keep` best groups are marked by +inf in their place, one after the other
@@ -153,7 +166,8 @@ moe_select_kernel(const float* __restrict__ logits, int n, const float* __restri
     }
     __syncthreads();
   }
-  if (live && lane < top) weights[(size_t)n_row * top + lane] = renormalize ? mine / sum : mine;
+  if (live && lane < top)
+    weights[(size_t)n_row * top + lane] = (renormalize ? mine / (sum + renormalize_eps) : mine) * weight_scale;
 }
 
 // ------------------------------------------------------------------------------------------------ align
@@ -503,10 +517,13 @@ int qil_moe_takes(int width, int outputs, int experts, int groups, int keep, int
 
 // x [n, width] (dtype), w_router float32 [outputs, width], bias and correction float32 [outputs] or null -> chosen
 // int32 [n, top], weights float32 [n, top].  logits: float32 scratch [n, outputs].
+// sigmoid_scores: scores are sigmoid(logit) instead of the softmax over all outputs.  group_top2: a group's score is
+// the sum of its two largest choice scores instead of its largest.  The weights are the chosen scores, divided by
+// (their sum + renormalize_eps) if renormalize, times weight_scale.
 int qil_moe_route(const void* x, int dtype, const float* w_router, const float* bias, const float* correction,
                   float* logits, int* chosen,
                   float* weights, int n, int width, int outputs, int groups, int keep, int top, int renormalize,
-                  hipStream_t s) {
+                  int sigmoid_scores, int group_top2, float weight_scale, float renormalize_eps, hipStream_t s) {
   if (n == 0) return 0;
   if (!qil_moe_takes(width, outputs, 0, groups, keep, top) || !logits) return -1;
   const dim3 g_logits((n + 7) / 8, (outputs + 3) / 4);
@@ -520,7 +537,8 @@ int qil_moe_route(const void* x, int dtype, const float* w_router, const float* 
   const int per_block = MOE_ROUTE_THREADS / QIL_WAVE;
   const size_t lds = (size_t)per_block * (2 * outputs + groups) * sizeof(float);
   hipLaunchKernelGGL(moe_select_kernel, dim3((n + per_block - 1) / per_block), dim3(MOE_ROUTE_THREADS), lds, s, logits, n,
-                     bias, correction, outputs, groups, keep, top, renormalize, chosen, weights);
+                     bias, correction, outputs, groups, keep, top, renormalize, chosen, weights, sigmoid_scores, group_top2,
+                     weight_scale, renormalize_eps);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -5,6 +5,12 @@
 #pragma once
 #include "common.h"
 
+// What a query at `position` is multiplied by when its temperature grows with the logarithm of the position:
+// 1 + coef * ln(floor((position + 1) / every) + 1); every <= 0: 1.
+__device__ __forceinline__ float query_temperature(int position, float coef, int every) {
+  return every > 0 ? 1.f + coef * logf((float)((position + 1) / every) + 1.f) : 1.f;
+}
+
 __device__ __forceinline__ void load8_sum(const float* base, size_t index, int splits, size_t stride, float* out) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) out[e] = 0.f;

@@ -38,11 +38,11 @@ __global__ void qk_norm_rope_store_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
     const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-    int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first) {
+    int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first, int row_elems,
+    float temp_coef, int temp_every) {
   __shared__ float vec[QIL_MAX_HEAD_DIM];
   const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int total_heads = heads + 2 * kv_heads;
-  const size_t src = ((size_t)n * total_heads + head) * d;        // index into qkv
+  const size_t src = (size_t)n * row_elems + (size_t)head * d;    // index into qkv
   const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
   if (!is_q && slots == nullptr) return;                 // a reader of another entry's cache writes no k/v
 
@@ -65,6 +65,7 @@ __global__ void qk_norm_rope_store_kernel(
   __syncthreads();
   const int half = rot / 2;
   const int position = positions[n];
+  const float temperature = is_q ? query_temperature(position, temp_coef, temp_every) : 1.f;
   const bool rotates = cos_table && rot > 0;
   // one element of the rotated head: from the tables, or (no sine table) from the frequencies the cosine table's place holds
   auto turned = [&](int i) {
@@ -88,7 +89,7 @@ __global__ void qk_norm_rope_store_kernel(
 #pragma unroll
     for (int u = 0; u < QIL_MAX_HEAD_DIM / QIL_WAVE; ++u) {
       const int i = lane + u * QIL_WAVE;
-      if (i < d) st(dst + i, weight ? round_to<T>(mine[u] * rstd) * weight[i] : mine[u]);
+      if (i < d) st(dst + i, (weight ? round_to<T>(mine[u] * rstd) * weight[i] : mine[u]) * temperature);
     }
     return;
   }
@@ -100,7 +101,7 @@ __global__ void qk_norm_rope_store_kernel(
     for (int i = lane; i < d; i += QIL_WAVE) vec[i] = round_to<T>(vec[i] * rstd) * weight[i];
     __syncthreads();
   }
-  for (int i = lane; i < d; i += QIL_WAVE) st(dst + i, turned(i));
+  for (int i = lane; i < d; i += QIL_WAVE) st(dst + i, turned(i) * temperature);
 }
 
 // The same work with eight consecutive elements a lane (16-byte vectors) and no LDS: a head is spread
@@ -115,7 +116,8 @@ qk_norm_rope_store_vec_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size,
-    float eps, int tg_log2, unsigned v_first_block, int norm_dim, int rotate_first) {
+    float eps, int tg_log2, unsigned v_first_block, int norm_dim, int rotate_first, int row_elems, float temp_coef,
+    int temp_every) {
   const int total_heads = heads + 2 * kv_heads;
   const int TG = 1 << tg_log2;
   if (blockIdx.x >= v_first_block) {
@@ -131,7 +133,7 @@ qk_norm_rope_store_vec_kernel(
     const int chunk = quad * 4 + (lane & 3);
     if (token >= (size_t)n) return;
     float x[8];
-    load8_sum(qkv, (token * total_heads + heads + kv_heads + kvh) * d + chunk * 8, splits, split_stride, x);
+    load8_sum(qkv, token * row_elems + (size_t)(heads + kv_heads + kvh) * d + chunk * 8, splits, split_stride, x);
     const int slot = slots[token];
     const size_t page = slot / page_size, offset = slot % page_size;
     T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + chunk * 8) * page_size + offset;
@@ -147,7 +149,7 @@ qk_norm_rope_store_vec_kernel(
   const bool is_q = head < heads, is_k = !is_q && head < heads + kv_heads;
   if (!is_q && slots == nullptr) return;
   float x[8];
-  load8_sum(qkv, ((size_t)token * total_heads + head) * d + chunk * 8, splits, split_stride, x);
+  load8_sum(qkv, (size_t)token * row_elems + (size_t)head * d + chunk * 8, splits, split_stride, x);
 
   if (!is_q && !is_k) {                                 // v: copy, transposed within the page
     const int kvh = head - heads - kv_heads, slot = slots[token];
@@ -160,6 +162,11 @@ qk_norm_rope_store_vec_kernel(
   norm_rope8<T>(x, chunk, TG, is_q ? q_weight : k_weight, norm_dim, eps, cos_table, sin_table, positions[token], rot,
                 rotate_first != 0);
   if (is_q) {
+    if (temp_every > 0) {
+      const float temperature = query_temperature(positions[token], temp_coef, temp_every);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= temperature;
+    }
     store8(q_out + ((size_t)token * heads + head) * d + chunk * 8, x);
   } else {
     const int kvh = head - heads, slot = slots[token];
@@ -173,17 +180,22 @@ qk_norm_rope_store_vec_kernel(
 // qkv: in_dtype QIL_BF16 (one array, splits == 1) or QIL_F32 ([splits][n][..] partial sums).  dtype: type
 // of q_out and of the caches.  norm_dim: the number of elements the head norm's mean runs over (0: d); smaller
 // than d when the heads are padded with zeros to a size the attention kernels take.
+// extra_columns: so many more columns follow the v heads in every row of qkv (another branch's part of a stacked
+// product); they are skipped.  kv_heads 0: the rows hold queries only (a reader of another entry's cache).
+// temp_every > 0: the query at position p is multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) last.
 extern "C" int qil_qk_norm_rope_store(
     const void* qkv, int in_dtype, int splits, void* q_out, const float* q_weight, const float* k_weight,
     const float* cos_table, const float* sin_table, const int* positions, const int* slots, void* k_cache,
     void* v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first,
-    int dtype, hipStream_t s) {
+    int extra_columns, float temp_coef, int temp_every, int dtype, hipStream_t s) {
   if (n == 0) return 0;
+  if (extra_columns < 0 || temp_every < 0 || kv_heads < 0 || (kv_heads == 0 && slots)) return -1;
+  const int row_elems = (heads + 2 * kv_heads) * d + extra_columns;
   if (norm_dim == 0) norm_dim = d;
   if (norm_dim < 1 || norm_dim > d) return -1;
   if (d > QIL_MAX_HEAD_DIM || rot > d || (rot & 1) || splits < 1 || (in_dtype == QIL_BF16 && splits != 1)) return -1;
   if (dtype == QIL_F32 && in_dtype != QIL_F32) return -1;
-  const size_t stride = (size_t)n * (heads + 2 * kv_heads) * d;
+  const size_t stride = (size_t)n * row_elems;
   dim3 grid(n, heads + 2 * kv_heads);
   // vector kernel: d / 8 a power of two up to 32, half of the rotated width a power-of-two number of chunks
   int tg_log2 = -1;
@@ -191,7 +203,8 @@ extern "C" int qil_qk_norm_rope_store(
     if (d == (8 << b)) tg_log2 = b;
   const int half_chunks = rot >> 4;
   const bool rot_fits = rot == 0 || !cos_table || (rot % 16 == 0 && (half_chunks & (half_chunks - 1)) == 0);
-  const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)q_weight | (uintptr_t)k_weight |
+  const bool aligned = row_elems % 8 == 0 &&
+                       (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)q_weight | (uintptr_t)k_weight |
                          (uintptr_t)cos_table | (uintptr_t)sin_table) % 16) == 0;
   if (tg_log2 > 0 && rot_fits && aligned) {
     // v in blocks of its own behind the others when a head has at least four chunks and there is a cache to write
@@ -204,7 +217,8 @@ extern "C" int qil_qk_norm_rope_store(
 #define QIL_QKV_CASE(TD, T)                                                                                           \
   hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)qkv, splits,    \
                      stride, (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache,       \
-                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block, norm_dim, rotate_first)
+                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block, norm_dim, rotate_first,       \
+                     row_elems, temp_coef, temp_every)
     if (dtype == QIL_F32) QIL_QKV_CASE(float, float);
     else if (in_dtype == QIL_F32) QIL_QKV_CASE(float, bf16_t);
     else QIL_QKV_CASE(bf16_t, bf16_t);
@@ -214,7 +228,7 @@ extern "C" int qil_qk_norm_rope_store(
 #define QIL_QK_CASE(TD, T)                                                                                            \
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TD, T>), grid, dim3(QIL_WAVE), 0, s, (const TD*)qkv, splits, stride,   \
                      (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache, (T*)v_cache,  \
-                     heads, kv_heads, d, rot, page_size, eps, norm_dim, rotate_first)
+                     heads, kv_heads, d, rot, page_size, eps, norm_dim, rotate_first, row_elems, temp_coef, temp_every)
   if (dtype == QIL_F32) QIL_QK_CASE(float, float);
   else if (in_dtype == QIL_F32) QIL_QK_CASE(float, bf16_t);
   else QIL_QK_CASE(bf16_t, bf16_t);

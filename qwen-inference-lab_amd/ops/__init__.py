@@ -112,7 +112,7 @@ class Unmerged:
     def merge(self):
         _check(library.load().qil_attn_merge(_ptr(self.workspace), _ptr(self.positions), None, _ptr(self.out),
                                              self.shape[0], self.heads, self.head_dim, self.window, self.part,
-                                             self.parts, _code(self.dtype), _stream()), 'attn_merge')
+                                             self.parts, _code(self.dtype), None, _stream()), 'attn_merge')
         return self.out
 
 
@@ -580,16 +580,22 @@ def _rotation_arguments(rotation, head_dim):
 
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False):
+                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False, extra_columns=0,
+                       q_temperature=None):
     """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given).  ``norm_dim``: the
     number of elements the norm's mean runs over when the heads are padded with zeros (default: head_dim).
     ``rotate_first``: the rotation comes before the norm.  A rotation that carries ``frequencies`` is applied from
     position * frequency, made in the kernel.
 
-    ``qkv`` [N, (heads + 2 kv_heads) d]: tensor of type ``dtype`` or Partials.  Returns q as ``dtype``
+    ``extra_columns``: so many more columns follow the v heads in every row of ``qkv`` (another branch of a stacked
+    product); they are skipped.  ``kv_heads`` 0: the rows hold queries only.  ``q_temperature`` (coef, every): the
+    query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) last, in float32.
+
+    ``qkv`` [N, (heads + 2 kv_heads) d + extra_columns]: tensor of type ``dtype`` or Partials.  Returns q as ``dtype``
     [N, heads * d]; k and v go into the caches at ``slots`` (None: not stored)."""
     n = qkv.shape[0]
-    pointer, code, splits = _operand(qkv, 'qkv', dtype, (n, (heads + 2 * kv_heads) * head_dim))
+    pointer, code, splits = _operand(qkv, 'qkv', dtype, (n, (heads + 2 * kv_heads) * head_dim + extra_columns))
+    coef, every = q_temperature if q_temperature is not None else (0.0, 0)
     _require(positions, 'positions', torch.int32, (n,))
     for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
         if w is not None:
@@ -604,7 +610,8 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
     _check(library.load().qil_qk_norm_rope_store(
         pointer, code, splits, _ptr(q), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions),
         _ptr(slots), _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps),
-        int(norm_dim or 0), int(bool(rotate_first)), _code(dtype), _stream()), 'qk_norm_rope_store')
+        int(norm_dim or 0), int(bool(rotate_first)), int(extra_columns), float(coef), int(every), _code(dtype), _stream()),
+        'qk_norm_rope_store')
     return q
 
 
@@ -723,7 +730,7 @@ def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, pag
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False, tile_seqs=None, softcap=None):
+                    unmerged=False, tile_seqs=None, softcap=None, sinks=None):
     """Attention of every row of the step over its request's cached keys.
 
     ``q`` [N, heads * head_dim] (head h at columns [h d, (h + 1) d)).  Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
@@ -737,8 +744,15 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
     kernel then gets blocks for these only (None: for every sequence; those of one row leave at once).
     ``softcap`` c: scores are scaled, then capped softly, c * tanh(score / c), before the softmax.  The kernels
     specialised for bfloat16 heads of 64 and 128 have no cap; capped steps run on the general tile kernel.
+    ``sinks`` float32 [heads]: exp(sinks[h]) joins the divisor of head h's softmax once (no key, no value, not
+    scaled).  It enters where a row's result is normalised: in the kernel when the keys are in one piece, in the merge
+    of the parts otherwise.  The general tile kernel, the matrix-core decode kernel and the row kernel take it; steps
+    with sinks run on those and come back merged.
     """
     cap = float(softcap or 0.0)
+    if sinks is not None:
+        _require(sinks, 'sinks', torch.float32, (heads,))
+        unmerged = False
     if cap < 0:
         raise ValueError('softcap must be positive')
     n = q.shape[0]
@@ -768,7 +782,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                 raise ValueError('tile_seqs must count the sequences of two or more rows')
             n_seqs = tile_seqs
         part, parts = tile_key_parts(lib, qkv.dtype, several, max_query, heads, kv_heads,
-                                     head_dim, page_size, block_tables.shape[1], max_context, general=cap > 0)
+                                     head_dim, page_size, block_tables.shape[1], max_context,
+                                     general=cap > 0 or sinks is not None)
         if parts > 1:
             # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
             # rows of the step: what the merge leaves in rows that are alone is overwritten below)
@@ -776,7 +791,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             merged = n if tile_seqs is None else n - single_rows.shape[0]
             workspace = torch.empty(lib.qil_attn_rows_workspace(merged, heads, head_dim, parts) // 4, dtype=torch.float32,
                                     device=qkv.device)
-            if cap == 0 and qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
+            if cap == 0 and sinks is None and qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
                     lib.qil_attn_tile_bf16_takes(head_dim, page_size, block_tables.shape[1]):
                 _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                     _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
@@ -790,12 +805,12 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                                                   kv_heads, head_dim, page_size, int(window or 0), float(scale), cap,
                                                   part, parts, _code(qkv.dtype), _stream()), 'attn_tile_in_parts')
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), merged, heads, head_dim,
-                                      int(window or 0), part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
+                                      int(window or 0), part, parts, _code(qkv.dtype), _ptr(sinks), _stream()), 'attn_merge')
         else:
             _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                      block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
                                      max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
-                                     cap, _code(qkv.dtype), _stream()), 'attn_tile')
+                                     cap, _code(qkv.dtype), _ptr(sinks), _stream()), 'attn_tile')
         rows = single_rows.shape[0]
     else:
         single_rows, rows = None, n
@@ -811,12 +826,12 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                                        _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
                                        window_arg, float(scale), part, parts, DECODE_WAVES,
                                        int(rows * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= 128), cap,
-                                       _stream()), 'attn_decode')
+                                       _ptr(sinks), _stream()), 'attn_decode')
             if unmerged and parts > 1 and single_rows is None:
                 return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
                                 part=part, parts=parts)
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), _ptr(single_rows), _ptr(out), rows, heads,
-                                      head_dim, window_arg, part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
+                                      head_dim, window_arg, part, parts, _code(qkv.dtype), _ptr(sinks), _stream()), 'attn_merge')
         else:
             part = _rows_part(rows, kv_heads, max_context)
             parts = max(1, -(-max_context // part))
@@ -833,7 +848,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                      block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                      _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
-                                     window_arg, float(scale), cap, part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
+                                     window_arg, float(scale), cap, part, parts, _code(qkv.dtype), _ptr(sinks), _stream()),
+                   'attn_rows')
     return out
 
 
@@ -1245,12 +1261,20 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
 
 # ---------------------------------------------------------------------------------------------------------------
 # Routed feed-forward
-def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None):
+ROUTER_SCORES = {'softmax': 0, 'sigmoid': 1}
+ROUTER_GROUP_SCORES = {'max': 0, 'top2': 1}
+
+
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None, score='softmax',
+              group_score='max', weight_scale=1.0, renormalize_eps=0.0):
     """x [N, width] (model type), router float32 [outputs, width], correction float32 [outputs] or None ->
     (chosen int32 [N, top], weights float32 [N, top]): softmax scores over all outputs in float32; the choice goes
     by score + correction among the outputs of the ``keep`` best of ``groups`` equal groups of neighbours (a group's
     score: its best choice score); the weights are the chosen outputs' scores (divided by their sum if asked, which
-    makes them the softmax over the chosen logits alone).  ``bias`` float32 [outputs]: added to the logits."""
+    makes them the softmax over the chosen logits alone).  ``bias`` float32 [outputs]: added to the logits.
+    ``score='sigmoid'``: scores are sigmoid(logit) and the choice goes by the score (+ correction);
+    ``group_score='top2'``: a group's score is the sum of its two largest choice scores; with ``renormalize`` the
+    divisor is the chosen scores' sum + ``renormalize_eps``; ``weight_scale`` multiplies the weights last."""
     n, width = x.shape
     _require(x, 'x')
     outputs = router.shape[0]
@@ -1266,8 +1290,9 @@ def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bi
     weights = torch.empty((n, top), dtype=torch.float32, device=x.device)
     logits = torch.empty((n, outputs), dtype=torch.float32, device=x.device)
     _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(bias), _ptr(correction), _ptr(logits), _ptr(chosen),
-                             _ptr(weights), n, width, outputs, groups, keep, top, int(bool(renormalize)), _stream()),
-           'moe_route')
+                             _ptr(weights), n, width, outputs, groups, keep, top, int(bool(renormalize)),
+                             ROUTER_SCORES[score], ROUTER_GROUP_SCORES[group_score], float(weight_scale),
+                             float(renormalize_eps), _stream()), 'moe_route')
     return chosen, weights
 
 
@@ -1299,3 +1324,130 @@ def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alp
                                ff, experts, top, tile_rows, max_tiles, GATE_FUNCTIONS[activation], float(limit),
                                float(alpha), _stream()), 'moe_experts')
     return RoutedSum(x, y, chosen, weights, experts) if lazy else out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Small float32 steps between products, and the selective state-space mixer's two kernels
+def _any_operand(value, name, shape):
+    """(pointer, dtype code, splits) of an input that is a bfloat16 or float32 tensor or Partials."""
+    if isinstance(value, Partials):
+        _require(value.tensor, name, torch.float32, (value.splits, *shape))
+        return value.tensor.data_ptr(), 0, value.splits
+    _require(value, name, None, shape)
+    return value.data_ptr(), _code(value.dtype), 1
+
+
+def scaled_sum(a, b, a_scale, b_scale):
+    """a_scale * a + b_scale * b as float32 [N, H]; ``a`` and ``b`` are tensors (float32 or bfloat16) or Partials."""
+    n, width = a.shape
+    if tuple(b.shape) != (n, width):
+        raise ValueError(f'scaled_sum: {tuple(a.shape)} and {tuple(b.shape)}')
+    a = _plain_delta(a)
+    pa, ca, sa = _any_operand(a, 'a', (n, width))
+    pb, cb, sb = _any_operand(b, 'b', (n, width))
+    out = torch.empty((n, width), dtype=torch.float32, device=a.device)
+    _check(library.load().qil_scaled_sum(pa, ca, sa, pb, cb, sb, float(a_scale), float(b_scale), _ptr(out), n, width,
+                                         _stream()), 'scaled_sum')
+    return out
+
+
+def sigmoid_gate(x, source, *, offset):
+    """x * sigmoid(source[:, offset : offset + C]) for x [N, C] of the model's type; ``source`` [N, W] is a tensor of
+    that type or Partials (the stacked product whose last columns are the gate's logits).  The sigmoid and the
+    product are float32; one rounding."""
+    n, columns = x.shape
+    _require(x, 'x')
+    width = source.shape[1]
+    if source.shape[0] != n or offset < 0 or offset + columns > width:
+        raise ValueError('sigmoid_gate: the gate columns do not lie inside the source')
+    pointer, code, splits = _any_operand(source, 'source', (n, width))
+    out = torch.empty_like(x)
+    _check(library.load().qil_sigmoid_gate(_ptr(x), pointer, code, splits, width, int(offset), _ptr(out), n, columns,
+                                           _code(x.dtype), _stream()), 'sigmoid_gate')
+    return out
+
+
+def soft_cap(x, cap):
+    """cap * tanh(x / cap) of a float32 tensor, in place; returns it."""
+    _require(x, 'x', torch.float32)
+    _check(library.load().qil_soft_cap(_ptr(x), float(cap), x.numel(), _stream()), 'soft_cap')
+    return x
+
+
+def check_selective_scan_geometry(*, inner, state, taps):
+    """Sizes the selective scan's kernels take; called when the part is built."""
+    if not (inner >= 1 and 1 <= state <= 256 and 1 <= taps <= 64):
+        raise UnsupportedShape(f'selective scan: inner {inner}, state {state} (at most 256), {taps} taps (at most 64)')
+
+
+CONV_ACTIVATIONS = {None: 0, 'silu': 1}
+
+
+def channel_conv(x, weight, bias, *, columns, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, activation,
+                 out_dtype):
+    """act(bias + causal convolution over time) on the first ``columns`` columns of ``x`` [N, W] (tensor of the
+    model's type or Partials): out[t, c] = act(bias[c] + sum_j weight[j, c] * x[t - taps + 1 + j, c]) over the rows of
+    every sequence of the step and the taps - 1 inputs before them, which are the sequence's state (``state`` float32
+    [slots, taps - 1, columns]: read unless the sequence starts at position 0, and left holding the sequence's last
+    taps - 1 inputs).  ``weight`` float32 [taps, columns], ``bias`` float32 [columns] or None.  -> [N, columns] of
+    ``out_dtype``; float32 arithmetic, one rounding."""
+    n, width = x.shape
+    taps = weight.shape[0]
+    _require(weight, 'weight', torch.float32, (taps, columns))
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, (columns,))
+    if taps > 1:
+        _require(state, 'state', torch.float32)
+        if state.ndim != 3 or tuple(state.shape[1:]) != (taps - 1, columns):
+            raise ValueError(f'channel_conv: state must be [slots, {taps - 1}, {columns}]')
+    _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+    _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+    _require(seq_slots, 'seq_slots', torch.int32, (n_seqs,))
+    _require(row_seq, 'row_seq', torch.int32, (n,))
+    pointer, code, splits = _any_operand(x, 'x', (n, width))
+    out = torch.empty((n, columns), dtype=out_dtype, device=weight.device)
+    _check(library.load().qil_channel_conv(pointer, code, splits, width, _ptr(weight), _ptr(bias),
+                                           _ptr(state) if taps > 1 else None, _ptr(cu_seqlens), _ptr(seq_starts),
+                                           _ptr(seq_slots), _ptr(row_seq), _ptr(out), _code(out_dtype), n, columns, taps,
+                                           CONV_ACTIVATIONS[activation], _stream()), 'channel_conv')
+    return out
+
+
+def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seqlens, seq_starts, seq_slots, n_seqs,
+                   out_dtype):
+    """The selective scan over every sequence of the step, its rows in order:
+
+        step = softplus(dt[t, c] + dt_bias[c]);   S[c, n] <- exp(step * a[c, n]) * S[c, n] + step * u[t, c] * B[t, n]
+        y[t, c] = (sum_n S[c, n] * C[t, n] + d[c] * u[t, c]) * silu(z[t, c])
+
+    ``u`` [N, C] of the model's type; ``dt`` [N, C], ``bc`` [N, 2 n] (B then C) and ``gate`` [N, W] (z from column
+    ``gate_offset`` on) are tensors of that type or Partials; ``dt_bias``, ``d`` float32 [C], ``a`` float32 [C, n];
+    ``state`` float32 [slots, C, n]: read unless the sequence starts at position 0, and left holding S after the
+    sequence's last row.  Everything from the step size on is float32.  -> [N, C] of ``out_dtype``."""
+    n, channels = u.shape
+    states = a.shape[1]
+    _require(u, 'u', out_dtype)
+    _require(a, 'a', torch.float32, (channels, states))
+    _require(dt_bias, 'dt_bias', torch.float32, (channels,))
+    _require(d, 'd', torch.float32, (channels,))
+    _require(state, 'state', torch.float32)
+    if state.ndim != 3 or tuple(state.shape[1:]) != (channels, states):
+        raise ValueError(f'selective_scan: state must be [slots, {channels}, {states}]')
+    _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+    _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+    _require(seq_slots, 'seq_slots', torch.int32, (n_seqs,))
+    gate_columns = gate.shape[1]
+    if gate_offset < 0 or gate_offset + channels > gate_columns:
+        raise ValueError('selective_scan: the gate columns do not lie inside their source')
+    p_dt, c_dt, s_dt = _any_operand(dt, 'dt', (n, channels))
+    p_bc, c_bc, s_bc = _any_operand(bc, 'bc', (n, 2 * states))
+    p_g, c_g, s_g = _any_operand(gate, 'gate', (n, gate_columns))
+    lib = library.load()
+    if not lib.qil_selective_scan_takes(channels, states, 1):
+        raise UnsupportedShape(f'selective_scan: {channels} channels of {states} states')
+    y = torch.empty((n, channels), dtype=out_dtype, device=u.device)
+    _check(lib.qil_selective_scan(_ptr(u), p_dt, c_dt, s_dt, _ptr(dt_bias), _ptr(a), p_bc, c_bc, s_bc, _ptr(d), p_g, c_g,
+                                  s_g, gate_columns, int(gate_offset), _ptr(state), _ptr(cu_seqlens), _ptr(seq_starts),
+                                  _ptr(seq_slots), _ptr(y), _code(out_dtype), n, n_seqs, channels, states, _stream()),
+           'selective_scan')
+    return y

@@ -212,18 +212,18 @@ def _declare(lib):
     lib.qil_add_rmsnorm.argtypes = [p, p, i, i, i, p, p, p, i, i, f, i, i, p]
     lib.qil_silu_mul.argtypes = [p, i, i, p, i, i, i, i, p]
     lib.qil_add_bias.argtypes = [p, p, i, i, i, p]
-    lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, f, i, i, p]
     lib.qil_attn_rows_workspace.argtypes = [i, i, i, i]
     lib.qil_attn_rows_workspace.restype = z
-    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, f, i, i, i, p]
-    lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, f, i, i, i, p, p]
+    lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p, p]
     lib.qil_attn_decode_fused_takes.argtypes = [i, i, i, i, i]
     lib.qil_attn_decode_fused_takes.restype = i
     lib.qil_attn_decode_fused.argtypes = [p, i, p, p, f, p, p, i, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, i, f, p]
     lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
     lib.qil_attn_decode_takes.restype = i
-    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, f, p]
-    lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, f, i, p]
+    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, f, p, p]
+    lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, f, i, p, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_splits.argtypes = [i, i, i]
     lib.qil_gemm_f32_waves.argtypes = [i, i, i, i]
@@ -325,8 +325,17 @@ def _declare(lib):
     lib.qil_moe_combine.restype = i
     lib.qil_moe_takes.argtypes = [i, i, i, i, i, i]
     lib.qil_moe_takes.restype = i
-    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, f, f, p]
     lib.qil_moe_route.restype = i
+    lib.qil_scaled_sum.argtypes = [p, i, i, p, i, i, f, f, p, i, i, p]
+    lib.qil_sigmoid_gate.argtypes = [p, p, i, i, i, i, p, i, i, i, p]
+    lib.qil_soft_cap.argtypes = [p, f, z, p]
+    lib.qil_channel_conv.argtypes = [p, i, i, i, p, p, p, p, p, p, p, p, i, i, i, i, i, p]
+    lib.qil_selective_scan_takes.argtypes = [i, i, i]
+    lib.qil_selective_scan.argtypes = [p, p, i, i, p, p, p, i, i, p, p, i, i, i, i, p, p, p, p, p, i, i, i, i, i, p]
+    for name in ('qil_scaled_sum', 'qil_sigmoid_gate', 'qil_soft_cap', 'qil_channel_conv', 'qil_selective_scan_takes',
+                 'qil_selective_scan'):
+        getattr(lib, name).restype = i
     lib.qil_moe_tile_rows.argtypes = [i, i]
     lib.qil_moe_tile_rows.restype = i
     lib.qil_moe_max_tiles.argtypes = [i, i, i]

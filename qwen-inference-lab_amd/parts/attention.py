@@ -30,13 +30,22 @@ class Attention(Mixer):
     declares no norm tensors); ``norm_after_rotation`` (queries and keys are rotated first and normed then).
     ``position`` may be a ``Rotary`` (tables) or a ``RotaryFrequencies`` (the kernels make the angles from the
     positions, which no table bounds).
+    ``out_bias``: whether the output projection has a bias (default: as ``bias``).
+    ``q_temperature`` (coef, every): the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)
+    after the head norm, in float32.
+    ``sink``: a stored number per query head (tensor ``sinks``) whose exponential joins the softmax's denominator
+    once: it has no key and no value and is not scaled.
+    ``gate``: the heads' results are multiplied element by element by sigmoid(W_g h) before the output projection
+    (tensor ``g_proj.weight`` [heads * value_dim, width], stacked under q/k/v: one product makes all four).
+    ``own_kv=False``: the part has no key and value projections; its schedule entry reads another entry's cache
+    (``ScheduleEntry.cache_of``), with its own queries, mask and everything else.
     """
     graph_safe = True
     takes_lazy_norm = True       # h goes into ops.linear only, which takes a norm not computed yet
 
     def __init__(self, *, width, heads, kv_heads, head_dim, bias, qk_norm_eps, scale,
                  position=None, window=None, dtype=torch.bfloat16, value_dim=None, softcap=None, qk_norm_weights=True,
-                 norm_after_rotation=False):
+                 norm_after_rotation=False, out_bias=None, q_temperature=None, sink=False, gate=False, own_kv=True):
         super().__init__()
         if heads % kv_heads:
             raise ValueError('heads must be a multiple of kv_heads')
@@ -46,6 +55,14 @@ class Attention(Mixer):
         self.value_dim = head_dim if value_dim is None else value_dim
         self.softcap = None if softcap is None else float(softcap)
         self.qk_norm_weights, self.norm_after_rotation = bool(qk_norm_weights), bool(norm_after_rotation)
+        self.out_bias = self.bias if out_bias is None else bool(out_bias)
+        self.sink, self.gate, self.own_kv = bool(sink), bool(gate), bool(own_kv)
+        self.q_temperature = None
+        if q_temperature is not None:
+            coef, every = q_temperature
+            if type(every) is not int or every < 1:
+                raise ValueError('the query temperature grows every so many positions: a positive integer')
+            self.q_temperature = (float(coef), every)
         if self.softcap is not None and not self.softcap > 0:
             raise ValueError('softcap must be positive')
         if type(self.value_dim) is not int or self.value_dim < 1:
@@ -60,14 +77,23 @@ class Attention(Mixer):
     def param_specs(self):
         q, kv, d = self.heads * self.head_dim, self.kv_heads * self.head_dim, self.head_dim
         v, o = self.kv_heads * self.value_dim, self.heads * self.value_dim
-        specs = {'q_proj.weight': ParamSpec((q, self.width)), 'k_proj.weight': ParamSpec((kv, self.width)),
-                 'v_proj.weight': ParamSpec((v, self.width)), 'o_proj.weight': ParamSpec((self.width, o))}
-        if self.bias:   # o_proj gets a bias too (qil/model.py:35)
-            specs.update({'q_proj.bias': ParamSpec((q,), 'vector'), 'k_proj.bias': ParamSpec((kv,), 'vector'),
-                          'v_proj.bias': ParamSpec((v,), 'vector'), 'o_proj.bias': ParamSpec((self.width,), 'vector')})
+        specs = {'q_proj.weight': ParamSpec((q, self.width)), 'o_proj.weight': ParamSpec((self.width, o))}
+        if self.own_kv:
+            specs.update({'k_proj.weight': ParamSpec((kv, self.width)), 'v_proj.weight': ParamSpec((v, self.width))})
+        if self.bias:
+            specs['q_proj.bias'] = ParamSpec((q,), 'vector')
+            if self.own_kv:
+                specs.update({'k_proj.bias': ParamSpec((kv,), 'vector'), 'v_proj.bias': ParamSpec((v,), 'vector')})
+        if self.out_bias:   # o_proj gets a bias too (qil/model.py:35)
+            specs['o_proj.bias'] = ParamSpec((self.width,), 'vector')
         if self.qk_norm_eps is not None and self.qk_norm_weights:
-            specs.update({'q_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal'),
-                          'k_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal')})
+            specs['q_norm.weight'] = ParamSpec((d,), 'vector', 'one_plus_normal')
+            if self.own_kv:
+                specs['k_norm.weight'] = ParamSpec((d,), 'vector', 'one_plus_normal')
+        if self.gate:
+            specs['g_proj.weight'] = ParamSpec((o, self.width))
+        if self.sink:
+            specs['sinks'] = ParamSpec((self.heads,), 'vector')
         return specs
 
     def cache_need(self):
@@ -91,12 +117,17 @@ class Attention(Mixer):
 
     def finalize(self):
         p = self.p
-        sizes = (self.head_dim, self.head_dim, self.value_dim)
-        self.w_qkv = torch.cat([self._pad_heads(p.pop(name), d=d) for name, d in
-                                zip(('q_proj.weight', 'k_proj.weight', 'v_proj.weight'), sizes)]).contiguous()
-        self.b_qkv = (torch.cat([self._pad_heads(p.pop(name), d=d) for name, d in
-                                 zip(('q_proj.bias', 'k_proj.bias', 'v_proj.bias'), sizes)]).contiguous()
-                      if self.bias else None)
+        stacked = [('q_proj', self.head_dim)]
+        if self.own_kv:
+            stacked += [('k_proj', self.head_dim), ('v_proj', self.value_dim)]
+        matrices = [self._pad_heads(p.pop(f'{name}.weight'), d=d) for name, d in stacked]
+        biases = [self._pad_heads(p.pop(f'{name}.bias'), d=d) for name, d in stacked] if self.bias else None
+        if self.gate:                                    # the gate's rows come last and have no bias
+            matrices.append(self._pad_heads(p.pop('g_proj.weight'), d=self.value_dim))
+            if self.bias:
+                biases.append(biases[0].new_zeros(self.heads * self.padded_dim))
+        self.w_qkv = torch.cat(matrices).contiguous()
+        self.b_qkv = torch.cat(biases).contiguous() if self.bias else None
         p['qkv_proj.weight'] = self.w_qkv
         if self.bias:
             p['qkv_proj.bias'] = self.b_qkv
@@ -113,14 +144,19 @@ class Attention(Mixer):
 
     def forward(self, h, ctx, cache):
         p = self.p
+        if cache.writes != self.own_kv:
+            raise ValueError('an attention part without keys and values of its own reads another entry\'s cache, '
+                             'and one with them writes its own')
         qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
         if self.qk_norm_eps is not None and not self.qk_norm_weights:
             norms = dict(q_weight=self._ones, k_weight=self._ones, eps=self.qk_norm_eps)
         else:
-            norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
+            norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight', p.get('q_norm.weight')),
                          eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
         sizes = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.padded_dim)
+        if self.gate or self.sink or self.q_temperature is not None or not self.own_kv:
+            return self._forward_extended(qkv, rotation, norms, sizes, ctx, cache)
         # (the kernel that makes its queries itself norms over the whole head it sees: not for padded heads)
         if ctx.max_query == 1 and self.padded_dim == self.head_dim and \
                 ops.decode_attention_takes(qkv, page_size=cache.page_size, rotation=rotation, dtype=self.dtype, **sizes):
@@ -141,4 +177,26 @@ class Attention(Mixer):
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
             max_query=ctx.max_query, max_context=ctx.max_context, tile_seqs=ctx.tile_seqs,
             scale=self.scale, window=self.window, unmerged=True, softcap=self.softcap, **sizes)
+        return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)
+
+    def _forward_extended(self, qkv, rotation, norms, sizes, ctx, cache):
+        """The step of a part with a query temperature, sinks, an output gate or another entry's keys and values:
+        the q/k kernel skips the gate's columns of the stacked product (and finds no key and value columns when the
+        part has none), the attention kernels take the sinks, and the gate multiplies what they return."""
+        p = self.p
+        gate_columns = self.heads * self.padded_dim if self.gate else 0
+        stored = self.kv_heads if self.own_kv else 0
+        q = ops.qk_norm_rope_store(
+            qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,
+            k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype, norm_dim=self.head_dim,
+            rotate_first=self.norm_after_rotation, heads=self.heads, kv_heads=stored, head_dim=self.padded_dim,
+            extra_columns=gate_columns, q_temperature=self.q_temperature, **norms)
+        attended = ops.paged_attention(
+            q, k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
+            block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
+            cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
+            max_query=ctx.max_query, max_context=ctx.max_context, tile_seqs=ctx.tile_seqs,
+            scale=self.scale, window=self.window, unmerged=False, softcap=self.softcap, sinks=p.get('sinks'), **sizes)
+        if self.gate:
+            attended = ops.sigmoid_gate(attended, qkv, offset=(self.heads + 2 * stored) * self.padded_dim)
         return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

@@ -27,11 +27,15 @@ class LMHead(Part):
 
     ``tied_to`` names an Embedding whose table is the head's matrix too
     (qil/model.py:96-98); the head then declares no tensor of its own.
+    ``softcap`` c: the logits become c * tanh(logits / c), in float32.
     """
 
-    def __init__(self, vocab, width, tied_to=None):
+    def __init__(self, vocab, width, tied_to=None, softcap=None):
         super().__init__()
         self.vocab, self.width, self.tied_to = vocab, width, tied_to
+        self.softcap = None if softcap is None else float(softcap)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError('softcap must be positive')
 
     def param_specs(self):
         return {} if self.tied_to is not None else {'weight': ParamSpec((self.vocab, self.width))}
@@ -42,4 +46,5 @@ class LMHead(Part):
 
     def forward(self, rows):
         import torch
-        return ops.linear(rows, self.weight, None, out_dtype=torch.float32)
+        logits = ops.linear(rows, self.weight, None, out_dtype=torch.float32)
+        return logits if self.softcap is None else ops.soft_cap(logits, self.softcap)

@@ -17,13 +17,21 @@ class RoutedExperts(FeedForward):
     (which makes them the softmax over the chosen logits alone).
     The result is the weighted sum of the chosen experts' outputs, in float32.
 
+    ``score='sigmoid'``: the scores are sigmoid(logit), each output by itself, instead of the softmax; the choice then
+    goes by the score (+ correction).  ``group_score='top2'``: a group's score is the sum of its two largest choice
+    scores instead of its largest.  With ``renormalize`` the chosen scores are divided by their sum +
+    ``renormalize_eps``; ``weight_scale`` multiplies the weights last.
+    ``shared``: a feed-forward part that every token passes and whose result is added to the routed sum (in float32,
+    by one kernel); its tensors are this part's own under the prefix ``shared.``.
+
     The experts' matrices are stacked at ``finalize`` into [experts, 2, ff, width] (gate rows, then up rows) and
     [experts, width, ff], ff padded with zeros to a multiple of 16 (a zero gate and up row give act = 0, which meets a
     zero column of the down matrix): pure re-layouts.
     """
 
     def __init__(self, *, width, experts, identity=0, top, groups=1, keep=1, intermediate, activation='silu', limit=None,
-                 alpha=1.0, correction=False, renormalize=False, bias=False, dtype=torch.bfloat16):
+                 alpha=1.0, correction=False, renormalize=False, bias=False, dtype=torch.bfloat16, score='softmax',
+                 group_score='max', weight_scale=1.0, renormalize_eps=0.0, shared=None):
         super().__init__()
         for name, value in (('experts', experts), ('top', top), ('groups', groups), ('keep', keep),
                             ('intermediate', intermediate)):
@@ -42,6 +50,18 @@ class RoutedExperts(FeedForward):
         self.outputs, self.intermediate, self.activation = outputs, intermediate, activation
         self.limit, self.alpha, self.correction, self.renormalize = float(limit or 0.0), float(alpha), bool(correction), bool(renormalize)
         self.dtype, self.bias = dtype, bool(bias)
+        if score not in ops.ROUTER_SCORES or group_score not in ops.ROUTER_GROUP_SCORES:
+            raise ValueError(f'no router kernel for score {score!r} with group score {group_score!r}')
+        self.score, self.group_score = score, group_score
+        self.weight_scale, self.renormalize_eps, self.shared = float(weight_scale), float(renormalize_eps), shared
+
+    def set_param(self, name, tensor):
+        if name.startswith('shared.'):
+            return self.shared.set_param(name[len('shared.'):], tensor)
+        return super().set_param(name, tensor)
+
+    def parameter_bytes(self):
+        return super().parameter_bytes() + (self.shared.parameter_bytes() if self.shared is not None else 0)
 
     def param_specs(self):
         specs = {'router.weight': ParamSpec((self.outputs, self.width), 'vector')}
@@ -53,9 +73,13 @@ class RoutedExperts(FeedForward):
             specs[f'experts.{e}.gate_proj.weight'] = ParamSpec((self.intermediate, self.width))
             specs[f'experts.{e}.up_proj.weight'] = ParamSpec((self.intermediate, self.width))
             specs[f'experts.{e}.down_proj.weight'] = ParamSpec((self.width, self.intermediate))
+        if self.shared is not None:
+            specs.update({'shared.' + name: spec for name, spec in self.shared.param_specs().items()})
         return specs
 
     def finalize(self):
+        if self.shared is not None:
+            self.shared.finalize()
         p = self.p
         ff, padded = self.intermediate, -(-self.intermediate // 16) * 16
         first = p['experts.0.gate_proj.weight']
@@ -70,9 +94,13 @@ class RoutedExperts(FeedForward):
     def forward(self, h, add_to=None):
         p = self.p
         chosen, weights = ops.moe_route(h, p['router.weight'], p.get('router.correction'), groups=self.groups,
-                                        keep=self.keep, top=self.top, renormalize=self.renormalize, bias=p.get('router.bias'))
+                                        keep=self.keep, top=self.top, renormalize=self.renormalize, bias=p.get('router.bias'),
+                                        score=self.score, group_score=self.group_score, weight_scale=self.weight_scale,
+                                        renormalize_eps=self.renormalize_eps)
         out = ops.moe_experts(h, chosen, weights, p['experts.gate_up_proj.weight'], p['experts.down_proj.weight'],
-                              activation=self.activation, limit=self.limit, alpha=self.alpha, lazy=True)
+                              activation=self.activation, limit=self.limit, alpha=self.alpha, lazy=self.shared is None)
+        if self.shared is not None:                     # routed sum + the shared expert's result, float32
+            return ops.Partials(ops.scaled_sum(out, self.shared.forward(h), 1.0, 1.0).unsqueeze(0))
         if isinstance(out, ops.RoutedSum):              # the norm that follows makes the weighted sum as it loads the rows
             return out
         return ops.Partials(out.unsqueeze(0))           # complete float32 sums: one split

@@ -6,15 +6,21 @@ from .. import ops
 
 
 class RMSNorm(Norm):
-    """y = cast(x * rsqrt(mean(x^2) + eps)) * weight; weight multiplies as stored."""
+    """y = cast(x * rsqrt(mean(x^2) + eps)) * (offset + weight).  ``offset`` 0: the weight multiplies as stored;
+    ``offset`` 1: a weight that is stored around zero.  The sum is made once, in float32, at ``finalize`` (the stored
+    weights are float32 on the device whatever the model's type), so the kernels see one factor per channel."""
     centre = False
 
-    def __init__(self, width, eps):
+    def __init__(self, width, eps, offset=0.0):
         super().__init__()
-        self.width, self.eps = int(width), float(eps)
+        self.width, self.eps, self.offset = int(width), float(eps), float(offset)
 
     def param_specs(self):
-        return {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal')}
+        return {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal' if self.offset == 0.0 else 'normal')}
+
+    def finalize(self):
+        if self.offset != 0.0:
+            self.p['weight'] = (self.p['weight'] + self.offset).contiguous()
 
     def forward(self, stream, delta, out_dtype, delta_scale=1.0):
         if delta_scale != 1.0:                      # (the general kernel rounds once, after the weight)

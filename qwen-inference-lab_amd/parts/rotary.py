@@ -7,6 +7,8 @@ bfloat16 rounding edges of cos/sin (docs/OPTIMIZATION_DEBUG_LOG.md:23-33).  The
 tables stay float32 whatever the model's dtype.  Pairing is (i, i + rot_dim/2)
 (qil/model.py:42-46).
 """
+import math
+
 import torch
 
 from .base import PositionEncoding, Rotation
@@ -38,11 +40,19 @@ class Rotary(PositionEncoding):
 class RotaryFrequencies(PositionEncoding):
     """The rotation as its frequencies alone: f_i = base**(-2 i / rot_dim), i < rot_dim / 2, made in float64 and held
     in float32.  Kernels that take it make the angle position * f_i and its cosine and sine themselves, in float32,
-    so no table bounds the positions.  Pairing is (i, i + rot_dim / 2)."""
+    so no table bounds the positions.  Pairing is (i, i + rot_dim / 2).
 
-    def __init__(self, rot_dim, base, *, device='cpu'):
+    ``scaling`` (factor, low, high, original): long waves are slowed.  With the wavelength l = 2 pi / f, f stays where
+    l < original / high, becomes f / factor where l > original / low, and between the two is
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+
+    def __init__(self, rot_dim, base, *, device='cpu', scaling=None):
         super().__init__()
         self.rot_dim, self.base, self.device = int(rot_dim), float(base), device
+        self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
+        if self.scaling is not None and (len(self.scaling) != 4 or not all(v > 0 for v in self.scaling) or
+                                         not self.scaling[2] > self.scaling[1]):
+            raise ValueError('scaling is (factor, low, high, original), all positive, high above low')
         if self.rot_dim < 2 or self.rot_dim % 2:
             raise ValueError('rot_dim must be even and at least 2')
         if not self.base > 0:
@@ -52,8 +62,20 @@ class RotaryFrequencies(PositionEncoding):
     def rotation(self):
         return Rotation(None, None, self.rot_dim, self.frequencies())
 
+    def _scaled(self, f):
+        if self.scaling is None:
+            return f
+        factor, low, high, original = self.scaling
+        wavelength = 2.0 * math.pi / f
+        if wavelength < original / high:
+            return f
+        if wavelength > original / low:
+            return f / factor
+        s = (original / wavelength - low) / (high - low)
+        return (1.0 - s) * f / factor + s * f
+
     def frequencies(self):
         if self._frequencies is None:
-            values = [self.base ** (-2.0 * i / self.rot_dim) for i in range(self.rot_dim // 2)]
+            values = [self._scaled(self.base ** (-2.0 * i / self.rot_dim)) for i in range(self.rot_dim // 2)]
             self._frequencies = torch.tensor(values, dtype=torch.float64).to(torch.float32).to(self.device).contiguous()
         return self._frequencies

@@ -83,10 +83,11 @@ def silu_mul(gate_up, out_dtype=None, interleaved=False):
 
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False):
+                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False, extra_columns=0,
+                       q_temperature=None):
     qkv = _value(qkv)
     n, d = qkv.shape[0], head_dim
-    x = qkv.view(n, heads + 2 * kv_heads, d)
+    x = qkv[:, :(heads + 2 * kv_heads) * d].reshape(n, heads + 2 * kv_heads, d)
     q, k, v = x[:, :heads].to(torch.float32), x[:, heads:heads + kv_heads].to(torch.float32), x[:, heads + kv_heads:]
 
     def normed(t, weight):
@@ -114,12 +115,18 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
         page, offset = slots.long() // page_size, slots.long() % page_size
         k_cache[page, :, offset] = shape(k, k_weight)
         v_cache[page, :, :, offset] = v.to(dtype)        # V is [pages, kv_heads, d, page_size]
+    if q_temperature is not None:
+        coef, every = q_temperature
+        factor = 1.0 + coef * torch.log(torch.div(positions + 1, every, rounding_mode='floor').to(torch.float32) + 1.0)
+        # the factor multiplies in float32, before the one rounding of the stored query
+        plain = normed(turned(q), q_weight) if rotate_first else turned(normed(q, q_weight))
+        return (plain * factor[:, None, None]).to(dtype).reshape(n, heads * d)
     return shape(q, q_weight).reshape(n, heads * d)
 
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False, tile_seqs=None, softcap=None, accumulate=torch.float32):
+                    unmerged=False, tile_seqs=None, softcap=None, sinks=None, accumulate=torch.float32):
     n, d, g = q.shape[0], head_dim, heads // kv_heads
     qkv = q
     q = q.reshape(n, heads, d).to(accumulate)
@@ -136,6 +143,10 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         scores = torch.einsum('hd,jhd->hj', q[row], keys) * scale
         if softcap:
             scores = softcap * torch.tanh(scores / softcap)
+        if sinks is not None:                        # one more term in the divisor: no key, no value
+            scores = torch.cat([scores, sinks.to(accumulate)[:, None]], dim=-1)
+            out[row] = torch.einsum('hj,jhd->hd', torch.softmax(scores, dim=-1)[:, :-1], values)
+            continue
         out[row] = torch.einsum('hj,jhd->hd', torch.softmax(scores, dim=-1), values)
     return out.reshape(n, heads * d).to(qkv.dtype)
 
@@ -375,20 +386,29 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
     return (unit * (torch.sigmoid(g) if gate == 'sigmoid' else g * torch.sigmoid(g))).to(out_dtype)
 
 
-def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None):
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False, bias=None, score='softmax',
+              group_score='max', weight_scale=1.0, renormalize_eps=0.0):
     logits = x.to(torch.float32) @ router.t() + (bias if bias is not None else 0.0)
-    scores = torch.softmax(logits, dim=-1)
-    choice = scores + correction if correction is not None else logits.clone()
+    if score == 'sigmoid':
+        scores = torch.sigmoid(logits)
+        choice = scores + correction if correction is not None else scores.clone()
+    else:
+        scores = torch.softmax(logits, dim=-1)
+        choice = scores + correction if correction is not None else logits.clone()
     n, outputs = scores.shape
     if groups > 1 and keep < groups:
-        best = choice.view(n, groups, outputs // groups).max(dim=-1).values
+        by_group = choice.view(n, groups, outputs // groups)
+        if group_score == 'top2' and outputs // groups > 1:
+            best = by_group.topk(2, dim=-1).values.sum(dim=-1)
+        else:
+            best = by_group.max(dim=-1).values
         kept = torch.zeros_like(best, dtype=torch.bool).scatter_(1, best.topk(keep, dim=-1).indices, True)
         choice = choice.masked_fill(~kept.repeat_interleave(outputs // groups, dim=1), float('-inf'))
     chosen = choice.topk(top, dim=-1).indices
     weights = scores.gather(1, chosen)
     if renormalize:
-        weights = weights / weights.sum(dim=-1, keepdim=True)
-    return chosen.to(torch.int32), weights
+        weights = weights / (weights.sum(dim=-1, keepdim=True) + renormalize_eps)
+    return chosen.to(torch.int32), weights * weight_scale
 
 
 def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0, lazy=False):
@@ -409,7 +429,68 @@ def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alp
     return out
 
 
-ALL = dict(moe_route=moe_route, moe_experts=moe_experts, embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
+def scaled_sum(a, b, a_scale, b_scale):
+    if hasattr(a, 'materialize'):
+        a = a.materialize()
+    return a_scale * _value(a).to(torch.float32) + b_scale * _value(b).to(torch.float32)
+
+
+def sigmoid_gate(x, source, *, offset):
+    gate = _value(source)[:, offset:offset + x.shape[1]].to(torch.float32)
+    return (x.to(torch.float32) * torch.sigmoid(gate)).to(x.dtype)
+
+
+def soft_cap(x, cap):
+    return x.copy_(cap * torch.tanh(x / cap))
+
+
+def check_selective_scan_geometry(*, inner, state, taps):
+    pass
+
+
+def channel_conv(x, weight, bias, *, columns, state, cu_seqlens, seq_starts, seq_slots, row_seq, n_seqs, activation,
+                 out_dtype):
+    x = _value(x)[:, :columns].to(torch.float32)
+    taps, keep = weight.shape[0], weight.shape[0] - 1               # weight [taps, C]
+    out = torch.empty_like(x)
+    for s in range(n_seqs):
+        first, last, start = int(cu_seqlens[s]), int(cu_seqlens[s + 1]), int(seq_starts[s])
+        before = torch.zeros((keep, columns), dtype=torch.float32)
+        if keep and start > 0:
+            before = state[int(seq_slots[s])].clone()
+            before[:max(0, keep - start)] = 0.0                 # places before the sequence's start
+        inputs = torch.cat([before, x[first:last]])
+        rows = last - first
+        total = sum(weight[j] * inputs[j:j + rows] for j in range(taps))
+        if bias is not None:
+            total = total + bias
+        out[first:last] = total * torch.sigmoid(total) if activation == 'silu' else total
+        if keep:
+            state[int(seq_slots[s])] = inputs[-keep:]
+    return out.to(out_dtype)
+
+
+def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seqlens, seq_starts, seq_slots, n_seqs,
+                   out_dtype):
+    n, channels = u.shape
+    states = a.shape[1]
+    uf, dtf, bcf = u.to(torch.float32), _value(dt).to(torch.float32), _value(bc).to(torch.float32)
+    z = _value(gate)[:, gate_offset:gate_offset + channels].to(torch.float32)
+    step = torch.nn.functional.softplus(dtf + dt_bias, threshold=20.0)
+    y = torch.empty((n, channels), dtype=torch.float32)
+    for s in range(n_seqs):
+        first, last = int(cu_seqlens[s]), int(cu_seqlens[s + 1])
+        S = state[int(seq_slots[s])].clone() if int(seq_starts[s]) > 0 else torch.zeros((channels, states))
+        for t in range(first, last):
+            S = torch.exp(step[t][:, None] * a) * S + (step[t] * uf[t])[:, None] * bcf[t, :states][None, :]
+            y[t] = S @ bcf[t, states:] + d * uf[t]
+        state[int(seq_slots[s])] = S
+    return (y * z * torch.sigmoid(z)).to(out_dtype)
+
+
+ALL = dict(scaled_sum=scaled_sum, sigmoid_gate=sigmoid_gate, soft_cap=soft_cap, channel_conv=channel_conv,
+           selective_scan=selective_scan, check_selective_scan_geometry=check_selective_scan_geometry,
+           moe_route=moe_route, moe_experts=moe_experts, embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
            qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample,
            add_norm=add_norm, rows_norm=rows_norm, gated_act=gated_act, latent_prepare=latent_prepare, head_product=head_product,
            latent_query=latent_query, latent_attention=latent_attention, state_scan_slot=state_scan_slot, state_scan=state_scan,
