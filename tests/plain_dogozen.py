@@ -193,8 +193,10 @@ def route(h, w, p, f):
     return chosen, weights, margin
 
 
-def routed(h, w, p, f):
-    chosen, weights, _ = route(h, w, p, f)
+def routed(h, w, p, f, margins=None):
+    chosen, weights, margin = route(h, w, p, f)
+    if margins is not None:
+        margins.append(margin)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, g in zip(chosen[t].tolist(), weights[t]):
@@ -204,13 +206,15 @@ def routed(h, w, p, f):
     return out
 
 
-def feed_forward(h, w, p, f):
-    return gated(h, w, p) if f['kind'] == 'dense' else routed(h, w, p, f)
+def feed_forward(h, w, p, f, margins=None):
+    return gated(h, w, p) if f['kind'] == 'dense' else routed(h, w, p, f, margins)
 
 
-def forward(config, w, tokens, start=0, states=None, collect=None):
+def forward(config, w, tokens, start=0, states=None, collect=None, margins=None):
     """Logits [T, vocab] of ``tokens`` at positions start ..; ``states``: the list (one dict a layer) that earlier calls
-    for the same sequence left, or None.  ``collect``: a list that receives the residual stream after every layer."""
+    for the same sequence left, or None.  ``collect``: a list that receives the residual stream after every layer;
+    ``margins``: a list that receives, per routed layer, every token's smallest gap between what its router chose and
+    what it did not."""
     eps = config['norm']['eps']
     states = states if states is not None else [dict() for _ in config['layers']]
     x = w['embed'][torch.as_tensor(tokens)]
@@ -226,7 +230,7 @@ def forward(config, w, tokens, start=0, states=None, collect=None):
             mixed = parallel_mixer(h, positions, w, p + 'mix.', layer['mixer'], states[i])
         x = x + norm(mixed, w[p + 'norm1b'], eps)
         if layer['mlp'] is not None:
-            x = x + norm(feed_forward(norm(x, w[p + 'norm2'], eps), w, p + 'mlp.', layer['mlp']), w[p + 'norm2b'], eps)
+            x = x + norm(feed_forward(norm(x, w[p + 'norm2'], eps), w, p + 'mlp.', layer['mlp'], margins), w[p + 'norm2b'], eps)
         if collect is not None:
             collect.append(x.clone())
     logits = norm(x, w['final.norm'], eps) @ w['embed'].T
@@ -234,3 +238,123 @@ def forward(config, w, tokens, start=0, states=None, collect=None):
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return logits, states
+
+
+# ------------------------------------------------------------------------------------------------ making models
+def attention_layer(*, heads, kv_heads, dim, vdim, scale, q_temp=None, kv_from=None, mlp=None):
+    mixer = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if q_temp is not None:
+        mixer['q_temp'] = dict(coef=q_temp[0], every=q_temp[1])
+    if kv_from is not None:
+        mixer['kv_from'] = kv_from
+    return dict(type='attention', mixer=mixer, mlp=mlp)
+
+
+def parallel_layer(*, heads, kv_heads, dim, vdim, scale, window, rot_dims, base=10000.0, scaling=None, inner, state, conv,
+                   dt_rank, left_scale=1.0, right_scale=1.0, mlp=None):
+    rot = dict(base=base, dims=rot_dims)
+    if scaling is not None:
+        rot['scaling'] = dict(zip(('factor', 'low', 'high', 'original'), scaling))
+    left = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, rot=rot, mask=dict(size=window))
+    right = dict(inner=inner, state=state, conv=conv, dt_rank=dt_rank)
+    return dict(type='parallel', mixer=dict(left=left, right=right, left_scale=left_scale, right_scale=right_scale), mlp=mlp)
+
+
+def dense_mlp(ff):
+    return dict(kind='dense', ff=ff)
+
+
+def moe_mlp(*, ff, experts, top, scale=1.0, count=1, keep=1, shared=None):
+    out = dict(kind='moe', expert=dict(ff=ff), router=dict(experts=experts, top=top, scale=scale,
+                                                          groups=dict(count=count, keep=keep)))
+    if shared is not None:
+        out['shared'] = dict(ff=shared)
+    return out
+
+
+def make_config(layers, *, vocab, width, eps=1e-5, softcap=None):
+    out = dict(architecture='Dogozen', vocab=vocab, width=width, layers=layers, norm=dict(eps=eps))
+    if softcap is not None:
+        out['logit_softcap'] = softcap
+    return out
+
+
+def random_weights(config, seed, spread=1.0):
+    """float64 tensors whose values bfloat16 holds exactly, by checkpoint name."""
+    g = torch.Generator().manual_seed(seed)
+    width = config['width']
+    w = {}
+
+    def held(t):
+        return t.to(torch.bfloat16).to(F)
+
+    def matrix(name, rows, columns, gain=1.0):
+        w[name] = held(torch.randn(rows, columns, generator=g, dtype=F) * (gain * spread / math.sqrt(columns)))
+
+    def vector(name, size, std=0.1, mean=0.0):
+        w[name] = held(mean + std * torch.randn(size, generator=g, dtype=F))
+
+    def gated_tensors(p, ff):
+        matrix(p + 'gate', ff, width)
+        matrix(p + 'up', ff, width)
+        matrix(p + 'down', width, ff)
+
+    w['embed'] = held(torch.randn(config['vocab'], width, generator=g, dtype=F))
+    vector('final.norm', width)
+    for i, layer in enumerate(config['layers']):
+        p, m = f'l{i}.', layer['mixer']
+        for name in ('norm1', 'norm1b') + (('norm2', 'norm2b') if layer['mlp'] is not None else ()):
+            vector(p + name, width)
+        if layer['type'] == 'attention':
+            H, G, d, dv = m['heads'], m['kv_heads'], m['dim'], m['vdim']
+            matrix(p + 'mix.q', H * d, width)
+            vector(p + 'mix.q.b', H * d, 0.3)
+            if m.get('kv_from') is None:
+                matrix(p + 'mix.k', G * d, width)
+                vector(p + 'mix.k.b', G * d, 0.3)
+                matrix(p + 'mix.v', G * dv, width)
+                vector(p + 'mix.v.b', G * dv, 0.3)
+            matrix(p + 'mix.g', H * dv, width, 2.0)
+            matrix(p + 'mix.o', width, H * dv)
+        else:
+            a, r = m['left'], m['right']
+            H, G, d, dv = a['heads'], a['kv_heads'], a['dim'], a['vdim']
+            matrix(p + 'mix.left.q', H * d, width, 2.0)
+            matrix(p + 'mix.left.k', G * d, width, 2.0)
+            matrix(p + 'mix.left.v', G * dv, width)
+            vector(p + 'mix.left.sink', H, 1.0)
+            matrix(p + 'mix.left.o', width, H * dv)
+            inner, n, taps, rank = r['inner'], r['state'], r['conv'], r['dt_rank']
+            matrix(p + 'mix.right.in', 2 * inner, width)
+            w[p + 'mix.right.conv'] = held(torch.randn(inner, taps, generator=g, dtype=F) * 0.5)
+            vector(p + 'mix.right.conv.b', inner, 0.2)
+            matrix(p + 'mix.right.x', rank + 2 * n, inner, 1.5)
+            matrix(p + 'mix.right.dt', inner, rank)
+            vector(p + 'mix.right.dt.b', inner, 1.0, -1.0)
+            w[p + 'mix.right.A_log'] = held(torch.log(torch.rand(inner, n, generator=g, dtype=F) * 4.0 + 0.05))
+            vector(p + 'mix.right.D', inner, 0.5, 1.0)
+            matrix(p + 'mix.right.o', width, inner)
+        f = layer['mlp']
+        if f is None:
+            continue
+        if f['kind'] == 'dense':
+            gated_tensors(p + 'mlp.', f['ff'])
+            continue
+        matrix(p + 'mlp.router', f['router']['experts'], width, 3.0)
+        for e in range(f['router']['experts']):
+            gated_tensors(f'{p}mlp.e{e}.', f['expert']['ff'])
+        if f.get('shared') is not None:
+            gated_tensors(p + 'mlp.shared.', f['shared']['ff'])
+    return w
+
+
+def logits(tokens, weights, config, margins=None):
+    """Logits [T, vocab] of a whole sequence (``margins`` as in ``forward``)."""
+    return forward(config, weights, tokens, margins=margins)[0]
+
+
+def greedy(prompt, count, weights, config):
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(logits(tokens, weights, config)[-1].argmax()))
+    return tokens[len(prompt):]
