@@ -253,6 +253,38 @@ def zinesun_config(z, layers, vocab, window, kind='turns'):
                 norm=dict(eps=1e-5))
 
 
+def dogozen_config(z, layers, vocab, window, kind='turns'):
+    """`layers` layers of the Dogozen design: gated attention without a rotation (queries with a temperature) behind a
+    routed feed-forward (32 experts in 4 groups of which 2 are kept, 4 chosen, each a quarter of the dense one, and a
+    shared expert of that size), or windowed attention with sinks beside a selective scan (inner size twice the
+    width, 16 states, four taps) behind a dense gated feed-forward, or both in turns; every fourth attention layer of
+    the turns reads the keys and values of the one before it."""
+    attention = dict(heads=z['heads'], kv_heads=max(1, z['heads'] // 4), dim=z['dim'], vdim=z['dim'], scale=z['dim'] ** -0.5,
+                     q_temp=dict(coef=0.1, every=256))
+    left = dict(heads=z['heads'], kv_heads=max(1, z['heads'] // 4), dim=z['dim'], vdim=z['dim'], scale=z['dim'] ** -0.5,
+                rot=dict(base=10000.0, dims=z['rot_dim'], scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)),
+                mask=dict(size=window))
+    right = dict(inner=2 * z['width'], state=16, conv=4, dt_rank=z['width'] // 16)
+    dense = dict(kind='dense', ff=z['ff'])
+    routed = dict(kind='moe', expert=dict(ff=z['ff'] // 4), shared=dict(ff=z['ff'] // 4),
+                  router=dict(experts=32, top=4, scale=2.5, groups=dict(count=4, keep=2)))
+    gated = dict(type='attention', mixer=attention, mlp=routed)
+    both = dict(type='parallel', mixer=dict(left=left, right=right, left_scale=0.5, right_scale=0.5), mlp=dense)
+    if kind == 'turns':
+        made = [both if i % 2 == 0 else gated for i in range(layers)]
+        if layers >= 4:
+            made[3] = dict(gated, mixer=dict(attention, kv_from=1))
+    elif kind == 'attention':
+        made = [dict(gated, mlp=dense)] * layers
+    elif kind == 'attention-routed':
+        made = [gated] * layers
+    elif kind == 'window':
+        made = [dict(both, mixer=dict(both['mixer'], right_scale=0.5, right=dict(inner=16, state=1, conv=1, dt_rank=1)))] * layers
+    else:
+        made = [both] * layers
+    return dict(architecture='Dogozen', vocab=vocab, width=z['width'], layers=made, norm=dict(eps=1e-6), logit_softcap=30.0)
+
+
 def designs_phase(args, torch, dtype):
     """Prefill tokens a second and decode milliseconds a step of a design's models whose layers are all of one kind
     (and of its kinds in turns), beside dense Qwen3 of the same width, feed-forward, depth and attention heads."""
@@ -267,6 +299,15 @@ def designs_phase(args, torch, dtype):
                   for kind, name in (('turns', 'feed-forwards in turns'), ('dense', 'dense feed-forwards'), ('routed', 'routed feed-forwards'))}
         models[f'zinesun (dense feed-forwards, window {8 * args.design_window})'] = zinesun_config(z, layers, vocab, 8 * args.design_window, 'dense')
         models['fubapel (latent attention only)'] = dict(fubapel_config(z, layers, vocab), layers=[fubapel_config(z, 1, vocab)['layers'][0]] * layers)
+        models['gerivik (capped attention only)'] = dict(gerivik_config(z, layers, vocab), layers=[gerivik_config(z, 2, vocab)['layers'][1]] * layers)
+    elif args.design == 'dogozen':
+        # beside it the closest model of the engine: Gerivik's capped attention with the routed feed-forward (the same
+        # arrangement of norms, grouped-query attention of the same sizes, a routed feed-forward of the same sizes)
+        names = (('turns', 'kinds in turns'), ('attention', 'gated attention, dense feed-forwards'),
+                 ('attention-routed', 'gated attention, routed feed-forwards'),
+                 ('parallel', f'window {args.design_window} beside a scan, dense feed-forwards'),
+                 ('window', f'window {args.design_window} beside a scan of one channel group, dense feed-forwards'))
+        models = {f'dogozen ({name})': dogozen_config(z, layers, vocab, args.design_window, kind) for kind, name in names}
         models['gerivik (capped attention only)'] = dict(gerivik_config(z, layers, vocab), layers=[gerivik_config(z, 2, vocab)['layers'][1]] * layers)
     elif args.design == 'gerivik':
         mixed = gerivik_config(z, layers, vocab)
@@ -349,8 +390,8 @@ def main():
                              'attention kernels alone, at the reference\'s own shapes and at the benchmark\'s.  products: a layer\'s '
                              'matrix products at --prefill-tokens rows alone, GPU BLAS against own kernel.  designs: prefill and decode of the '
                              'design named by --design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
-    parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik', 'zinesun'], help='the design of --phase designs')
-    parser.add_argument('--design-window', type=int, default=512, help='the attention window of --design zinesun')
+    parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik', 'zinesun', 'dogozen'], help='the design of --phase designs')
+    parser.add_argument('--design-window', type=int, default=512, help='the attention window of --design zinesun and --design dogozen')
     parser.add_argument('--design-only', default=None, help='of the models of --phase designs, only those whose name holds this (for profiling)')
     parser.add_argument('--design-sizes', default='1b', choices=sorted(DESIGN_SIZES), help='layer sizes of --phase designs')
     parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')

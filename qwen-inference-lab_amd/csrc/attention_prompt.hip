@@ -58,7 +58,7 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
                    const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
                    int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift,
                    float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P,
-                   int parts, float softcap) {
+                   int parts, float softcap, const float* __restrict__ sinks) {
   const float raw_scale = scale;
   if (CAP) scale = 1.f;
   constexpr int D = PROMPT_D, BK = PROMPT_BK, THREADS = WAVES * QIL_WAVE;
@@ -424,7 +424,8 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
     }
     return;
   }
-  const float inv = 1.f / total;
+  // (sinks: one more term exp(sink) in the divisor, no key, no value; row_m is the exponents' reference of l and ow)
+  const float inv = (!SPLIT && sinks) ? sink_reciprocal(total, row_m * scale, sinks[head]) : 1.f / total;
   bf16_t* orow = out + ((size_t)(q0 + my_row) * heads + head) * D;
 #pragma unroll
   for (int t = 0; t < WTILES; ++t)
@@ -438,7 +439,8 @@ template <int WAVES, bool SPLIT = false, bool CAP = false>
 static int launch_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                          int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                          int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s,
-                         float* workspace, int total_rows, int P, int parts, float softcap = 0.f) {
+                         float* workspace, int total_rows, int P, int parts, float softcap = 0.f,
+                         const float* sinks = nullptr) {
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = (SPLIT ? WAVES / 2 : WAVES) / GH;
   const size_t lds = (SPLIT ? 4 : 2) * (size_t)PROMPT_TILE_BYTES + (size_t)table_stride * sizeof(int);
@@ -458,7 +460,7 @@ static int launch_prompt(const void* q, int q_stride, const void* k_cache, const
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                      (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
                      kv_heads, page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts,
-                     softcap);
+                     softcap, sinks);
   return (int)hipGetLastError();
 }
 
@@ -505,4 +507,17 @@ extern "C" int qil_attn_prompt_capped(const void* q, int q_stride, const void* k
   return launch_prompt<4, false, true>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
                                        out, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
                                        (float*)workspace, total_rows, P, parts, softcap);
+}
+
+// The same with sinks (float32 [heads]: exp(sink) joins every head's divisor once), keys in one part, blocks of 4 waves.
+extern "C" int qil_attn_prompt_sinks(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                     const int* block_tables, int table_stride, const int* cu_seqlens,
+                                     const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                     int page_size, int window, float scale, const float* sinks, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if (!qil_attn_prompt_takes(PROMPT_D, page_size, table_stride) || heads % kv_heads || n_seqs > 65535 ||
+      (long)kv_heads * 2 > 65535 || !sinks || !out)
+    return -1;
+  return launch_prompt<4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
+                          max_query, heads, kv_heads, page_size, window, scale, s, nullptr, 0, 0, 1, 0.f, sinks);
 }

@@ -565,6 +565,10 @@ extern "C" int qil_attn_tile_key_parts(int n_seqs, int max_query, int heads, int
 
 // Sequences with >= 2 rows.  q: rows of stride q_stride, head h at h * d; out [rows, heads * d].
 // Requires d % 8 == 0, 8 <= d <= 256.  Returns -1 on a size it does not take.
+extern "C" int qil_attn_prompt_sinks(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                     const int* block_tables, int table_stride, const int* cu_seqlens,
+                                     const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                     int page_size, int window, float scale, const float* sinks, hipStream_t s);
 // parts > 1: the keys in `parts` parts of P keys (P a multiple of 64) on this file's kernel; every row of a sequence
 // of two or more rows gets float32 partial results in `workspace` (qil_attn_rows_workspace bytes for all `total_rows`
 // rows of the step, indexed by the step's row) for qil_attn_merge, and `out` is not written.
@@ -580,6 +584,10 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
     return qil_attn_prompt_capped(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                                   n_seqs, max_query, heads, kv_heads, page_size, window, scale, softcap, workspace,
                                   total_rows, P, parts, s);
+  // sinks on bfloat16 heads of 128, keys in one part: the prompt kernel's form with sinks
+  if (sinks && parts == 1 && softcap <= 0.f && dtype == QIL_BF16 && qil_attn_prompt_takes(d, page_size, table_stride))
+    return qil_attn_prompt_sinks(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                 n_seqs, max_query, heads, kv_heads, page_size, window, scale, sinks, s);
   if (parts == 1 && softcap <= 0.f && !sinks && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
     return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);

@@ -746,8 +746,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
     specialised for bfloat16 heads of 64 and 128 have no cap; capped steps run on the general tile kernel.
     ``sinks`` float32 [heads]: exp(sinks[h]) joins the divisor of head h's softmax once (no key, no value, not
     scaled).  It enters where a row's result is normalised: in the kernel when the keys are in one piece, in the merge
-    of the parts otherwise.  The general tile kernel, the matrix-core decode kernel and the row kernel take it; steps
-    with sinks run on those and come back merged.
+    of the parts otherwise.  The general tile kernel, the bfloat16 prompt kernel for heads of 128, the matrix-core
+    decode kernel and the row kernel take it; steps with sinks run on those and come back merged.
     """
     cap = float(softcap or 0.0)
     if sinks is not None:
@@ -782,8 +782,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                 raise ValueError('tile_seqs must count the sequences of two or more rows')
             n_seqs = tile_seqs
         part, parts = tile_key_parts(lib, qkv.dtype, several, max_query, heads, kv_heads,
-                                     head_dim, page_size, block_tables.shape[1], max_context,
-                                     general=cap > 0 or sinks is not None)
+                                     head_dim, page_size, block_tables.shape[1], max_context, general=cap > 0)
         if parts > 1:
             # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
             # rows of the step: what the merge leaves in rows that are alone is overwritten below)
@@ -791,7 +790,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             merged = n if tile_seqs is None else n - single_rows.shape[0]
             workspace = torch.empty(lib.qil_attn_rows_workspace(merged, heads, head_dim, parts) // 4, dtype=torch.float32,
                                     device=qkv.device)
-            if cap == 0 and sinks is None and qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
+            if cap == 0 and qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
                     lib.qil_attn_tile_bf16_takes(head_dim, page_size, block_tables.shape[1]):
                 _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                     _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),

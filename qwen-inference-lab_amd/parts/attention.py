@@ -144,9 +144,8 @@ class Attention(Mixer):
 
     def forward(self, h, ctx, cache):
         p = self.p
-        if cache.writes != self.own_kv:
-            raise ValueError('an attention part without keys and values of its own reads another entry\'s cache, '
-                             'and one with them writes its own')
+        if cache.writes and not self.own_kv:
+            raise ValueError('an attention part without keys and values of its own reads another entry\'s cache')
         qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
         if self.qk_norm_eps is not None and not self.qk_norm_weights:

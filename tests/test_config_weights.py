@@ -13,7 +13,7 @@ from qil_amd.weights import WeightsError, load_model, write_random_model
 
 
 def test_registry_names_and_reads():
-    assert known_architectures() == ['Fubapel', 'Gerivik', 'Qwen3ForCausalLM', 'Zinesun']
+    assert known_architectures() == ['Dogozen', 'Fubapel', 'Gerivik', 'Qwen3ForCausalLM', 'Zinesun']
     entry = architecture_for(dict(plain.TINY_B))
     assert entry.config_class is Qwen3Config
     without_name = {k: v for k, v in plain.TINY_B.items() if k != 'architectures'}
