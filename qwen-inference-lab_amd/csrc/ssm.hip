@@ -18,6 +18,16 @@
 //    moves), lane l holds the states l, l + 16, ...; the sum over the states is four such moves.  The loads of a
 //    token do not depend on the state, so four tokens' loads go out before their updates run.
 //    Everything from dt on is float32; u, B, C, z and dt_raw come as the products left them.
+//
+//    Up to 32 states the scan runs with a thread a channel and the channel's states in registers
+//    (scan_chunk_kernel): no sum across lanes, dt and u are loaded once a channel and token in whole lines, and B and
+//    C, which all channels share, are staged in LDS a tile of 64 tokens at a time.  A step whose sequences bring at
+//    most 64 rows walks each from its stored state in one launch.  Longer portions are cut into chunks of 64 tokens
+//    that run side by side: the recurrence is linear in the state, S_end = P S_in + E with P = exp(A * sum of the
+//    chunk's dt) and E the chunk's end state from zero, so (1) every chunk is walked from zero and leaves E and its
+//    sum of dt, (2) a small kernel walks a sequence's chunks in order, leaves every chunk's S_in where its E was and
+//    the sequence's last state in its slot, (3) every chunk is walked again from its S_in and writes y.  The bfloat16
+//    model takes exp(dt A) as the hardware's exp2 of dt * (A log2 e); the float32 model calls expf.
 #include "common.h"
 #include "operand.h"
 
@@ -133,6 +143,130 @@ selective_scan_kernel(const T* __restrict__ u, Operand dt_raw, const float* __re
   }
 }
 
+
+#define SCAN_L 64                      // tokens a chunk, and a tile of B and C in LDS
+#define SCAN_THREADS 256
+
+template <bool FAST> __device__ __forceinline__ float scan_decay(float step, float rate) {
+  return FAST ? __builtin_amdgcn_exp2f(step * rate) : expf(step * rate);          // FAST: rate = A * log2(e)
+}
+template <bool FAST> __device__ __forceinline__ float scan_softplus(float v) {
+  if (v > 20.f) return v;
+  return FAST ? __logf(1.f + __expf(v)) : log1pf(expf(v));
+}
+template <bool FAST> __device__ __forceinline__ float scan_silu(float v) {
+  return FAST ? v * __builtin_amdgcn_rcpf(1.f + __expf(-v)) : v / (1.f + expf(-v));
+}
+
+// PHASE 0: a sequence's rows from its stored state, y and the new state written.  PHASE 1: a chunk from zero; its end
+// state goes to carry[seq * max_chunks + chunk][channel][NS] and its sum of steps to sums[..][channel].  PHASE 2: a
+// chunk from the state that the carry kernel left in carry[..]; y written.
+template <typename T, int NS, int PHASE>
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_chunk_kernel(const T* __restrict__ u, Operand dt_raw, const float* __restrict__ dt_bias,
+                  const float* __restrict__ a, Operand bc, const float* __restrict__ d, Operand gate, int gate_columns,
+                  int gate_offset, float* state, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts,
+                  const int* __restrict__ seq_slots, T* __restrict__ y, int channels, int states, float* carry,
+                  float* sums, int max_chunks) {
+  constexpr bool FAST = sizeof(T) == 2;
+  __shared__ float tile[SCAN_L * 2 * NS];
+  const int c = blockIdx.x * SCAN_THREADS + threadIdx.x, seq = blockIdx.y, chunk = PHASE == 0 ? 0 : blockIdx.z;
+  const bool live = c < channels;
+  const int cc = live ? c : channels - 1;              // threads past the end walk a copy and store nothing
+  int first = cu_seqlens[seq], last = cu_seqlens[seq + 1];
+  if (PHASE != 0) {
+    first += chunk * SCAN_L;
+    if (first >= last) return;                         // (the whole block)
+    last = min(last, first + SCAN_L);
+  }
+  const size_t cell = (size_t)seq * max_chunks + chunk;
+  float rate[NS], S[NS];
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const float an = n < states ? a[(size_t)cc * states + n] : 0.f;
+    rate[n] = FAST ? an * 1.44269504088896f : an;
+    S[n] = 0.f;
+  }
+  if (PHASE == 0 && seq_starts[seq] > 0) {
+    const float* held = state + ((size_t)seq_slots[seq] * channels + cc) * states;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) if (n < states) S[n] = held[n];
+  }
+  if (PHASE == 2) {
+#pragma unroll
+    for (int n = 0; n < NS; ++n) S[n] = carry[(cell * channels + cc) * NS + n];
+  }
+  const float bias = dt_bias[cc], skip = d[cc];
+  float total = 0.f;
+  for (int t0 = first; t0 < last; t0 += SCAN_L) {
+    const int rows = min(SCAN_L, last - t0);
+    __syncthreads();                                   // the tile before this one has been used
+    for (int i = threadIdx.x; i < rows * 2 * NS; i += SCAN_THREADS) {
+      const int r = i / (2 * NS), k = i - r * 2 * NS, half = k / NS, n = k - half * NS;
+      tile[i] = n < states ? operand_at(bc, (size_t)(t0 + r) * 2 * states + half * states + n) : 0.f;
+    }
+    __syncthreads();
+    for (int r0 = 0; r0 < rows; r0 += 8) {
+      float dt[8], uv[8], zv[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const size_t t = min(t0 + r0 + k, last - 1);
+        dt[k] = operand_at(dt_raw, t * channels + cc);
+        uv[k] = ld(u + t * channels + cc);
+        zv[k] = PHASE == 1 ? 0.f : operand_at(gate, t * gate_columns + gate_offset + cc);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (r0 + k < rows) {
+          const float step = scan_softplus<FAST>(dt[k] + bias), in = step * uv[k];
+          const float* B = tile + (r0 + k) * 2 * NS;
+          float acc = 0.f;
+#pragma unroll
+          for (int n = 0; n < NS; ++n) {
+            S[n] = scan_decay<FAST>(step, rate[n]) * S[n] + in * B[n];
+            if (PHASE != 1) acc += S[n] * B[NS + n];
+          }
+          if (PHASE == 1) total += step;
+          else if (live) st(y + (size_t)(t0 + r0 + k) * channels + c, (acc + skip * uv[k]) * scan_silu<FAST>(zv[k]));
+        }
+      }
+    }
+  }
+  if (!live) return;
+  if (PHASE == 0) {
+    float* held = state + ((size_t)seq_slots[seq] * channels + c) * states;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) if (n < states) held[n] = S[n];
+  }
+  if (PHASE == 1) {
+#pragma unroll
+    for (int n = 0; n < NS; ++n) carry[(cell * channels + c) * NS + n] = S[n];
+    sums[cell * channels + c] = total;
+  }
+}
+
+// A sequence's chunks in order, a thread a (channel, state): every chunk's end state from zero is replaced by the state
+// it starts from, and the sequence's last state goes to its slot.
+__global__ void scan_carry_kernel(float* carry, const float* __restrict__ sums, const float* __restrict__ a, float* state,
+                                  const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts,
+                                  const int* __restrict__ seq_slots, int channels, int states, int NS, int max_chunks) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x, seq = blockIdx.y;
+  if (i >= channels * states) return;
+  const int c = i / states, n = i - c * states;
+  const int chunks = (cu_seqlens[seq + 1] - cu_seqlens[seq] + SCAN_L - 1) / SCAN_L;
+  float* held = state + ((size_t)seq_slots[seq] * channels + c) * states + n;
+  float S = seq_starts[seq] > 0 ? *held : 0.f;
+  const float an = a[(size_t)c * states + n];
+  for (int chunk = 0; chunk < chunks; ++chunk) {
+    const size_t cell = (size_t)seq * max_chunks + chunk;
+    float* at = carry + (cell * channels + c) * NS + n;
+    const float end = *at;
+    *at = S;
+    S = expf(an * sums[cell * channels + c]) * S + end;
+  }
+  *held = S;
+}
+
 extern "C" {
 
 int qil_selective_scan_takes(int channels, int states, int taps) {
@@ -160,20 +294,60 @@ int qil_channel_conv(const void* x, int x_code, int x_splits, int x_columns, con
   QIL_RETURN_LAUNCH_STATUS();
 }
 
+// Bytes of float32 workspace the scan needs for a step whose longest sequence brings max_query rows (0: none).
+size_t qil_selective_scan_workspace(int n_seqs, int max_query, int channels, int states) {
+  const int chunks = (max_query + SCAN_L - 1) / SCAN_L;
+  if (states > 32 || chunks <= 1) return 0;
+  return (size_t)n_seqs * chunks * channels * ((states + 7) / 8 * 8 + 1) * sizeof(float);
+}
+
 // u, y: [n, channels] of dtype; dt_raw [n, channels], bc [n, 2 * states] (B then C), gate [n, gate_columns] with z from
 // column gate_offset on: each QIL_BF16, or QIL_F32 with so many partial sums; dt_bias, d float32 [channels]; a float32
-// [channels, states]; state float32 [slots][channels][states].
+// [channels, states]; state float32 [slots][channels][states].  max_query: the most rows of one sequence; workspace:
+// qil_selective_scan_workspace bytes (may be null when that is 0).
 int qil_selective_scan(const void* u, const void* dt_raw, int dt_code, int dt_splits, const float* dt_bias, const float* a,
                        const void* bc, int bc_code, int bc_splits, const float* d, const void* gate, int gate_code,
                        int gate_splits, int gate_columns, int gate_offset, float* state, const int* cu_seqlens,
                        const int* seq_starts, const int* seq_slots, void* y, int dtype, int n, int n_seqs, int channels,
-                       int states, hipStream_t s) {
+                       int states, int max_query, float* workspace, hipStream_t s) {
   if (n == 0 || n_seqs == 0) return 0;
   if (!qil_selective_scan_takes(channels, states, 1) || !state || gate_offset < 0 || gate_offset + channels > gate_columns ||
       dt_splits < 1 || bc_splits < 1 || gate_splits < 1 || (dt_code == QIL_BF16 && dt_splits != 1) ||
       (bc_code == QIL_BF16 && bc_splits != 1) || (gate_code == QIL_BF16 && gate_splits != 1) || n_seqs > 65535) return -1;
   const Operand odt{dt_raw, dt_code, dt_splits, (size_t)n * channels}, obc{bc, bc_code, bc_splits, (size_t)n * 2 * states},
       og{gate, gate_code, gate_splits, (size_t)n * gate_columns};
+  if (states <= 32) {                                  // a thread a channel, the states in registers
+    const int chunks = (max_query + SCAN_L - 1) / SCAN_L;
+    if (max_query < 1 || (chunks > 1 && !workspace) || chunks > 65535) return -1;
+    const dim3 blocks((channels + SCAN_THREADS - 1) / SCAN_THREADS, n_seqs, chunks);
+    float* carry = workspace;
+    const int ns = (states + 7) / 8 * 8;
+    float* sums = workspace ? workspace + (size_t)n_seqs * chunks * channels * ns : nullptr;
+#define QIL_CHUNK(T, NS, PHASE)                                                                                       \
+  hipLaunchKernelGGL((scan_chunk_kernel<T, NS, PHASE>), blocks, dim3(SCAN_THREADS), 0, s, (const T*)u, odt, dt_bias, a, \
+                     obc, d, og, gate_columns, gate_offset, state, cu_seqlens, seq_starts, seq_slots, (T*)y, channels,  \
+                     states, carry, sums, chunks)
+#define QIL_CHUNK_NS(T, PHASE)                                                                                        \
+  do {                                                                                                                \
+    if (ns == 8) QIL_CHUNK(T, 8, PHASE); else if (ns == 16) QIL_CHUNK(T, 16, PHASE);                                   \
+    else if (ns == 24) QIL_CHUNK(T, 24, PHASE); else QIL_CHUNK(T, 32, PHASE);                                          \
+  } while (0)
+#define QIL_CHUNK_T(PHASE)                                                                                            \
+  do { if (dtype == QIL_F32) QIL_CHUNK_NS(float, PHASE); else QIL_CHUNK_NS(bf16_t, PHASE); } while (0)
+    if (chunks == 1) {
+      QIL_CHUNK_T(0);
+      QIL_RETURN_LAUNCH_STATUS();
+    }
+    QIL_CHUNK_T(1);
+    const int pairs = channels * states;
+    hipLaunchKernelGGL(scan_carry_kernel, dim3((pairs + 255) / 256, n_seqs), dim3(256), 0, s, carry, sums, a, state,
+                       cu_seqlens, seq_starts, seq_slots, channels, states, ns, chunks);
+    QIL_CHUNK_T(2);
+#undef QIL_CHUNK_T
+#undef QIL_CHUNK_NS
+#undef QIL_CHUNK
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   const dim3 grid((channels + 15) / 16, n_seqs);
   const int per = (states + 15) / 16;
 #define QIL_SCAN(T, NPER)                                                                                             \

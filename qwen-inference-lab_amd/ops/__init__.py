@@ -1413,7 +1413,7 @@ def channel_conv(x, weight, bias, *, columns, state, cu_seqlens, seq_starts, seq
 
 
 def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seqlens, seq_starts, seq_slots, n_seqs,
-                   out_dtype):
+                   max_query, out_dtype):
     """The selective scan over every sequence of the step, its rows in order:
 
         step = softplus(dt[t, c] + dt_bias[c]);   S[c, n] <- exp(step * a[c, n]) * S[c, n] + step * u[t, c] * B[t, n]
@@ -1422,7 +1422,10 @@ def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seq
     ``u`` [N, C] of the model's type; ``dt`` [N, C], ``bc`` [N, 2 n] (B then C) and ``gate`` [N, W] (z from column
     ``gate_offset`` on) are tensors of that type or Partials; ``dt_bias``, ``d`` float32 [C], ``a`` float32 [C, n];
     ``state`` float32 [slots, C, n]: read unless the sequence starts at position 0, and left holding S after the
-    sequence's last row.  Everything from the step size on is float32.  -> [N, C] of ``out_dtype``."""
+    sequence's last row.  Everything from the step size on is float32.  -> [N, C] of ``out_dtype``.
+    ``max_query``: the most rows of one sequence.  Up to 32 states a thread takes a channel with its states in
+    registers; sequences of more than 64 rows are then cut into chunks of 64 tokens that run side by side (every chunk
+    from zero, a carry over the chunks, every chunk again from its true state).  The forms differ by rounding only."""
     n, channels = u.shape
     states = a.shape[1]
     _require(u, 'u', out_dtype)
@@ -1445,8 +1448,10 @@ def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seq
     if not lib.qil_selective_scan_takes(channels, states, 1):
         raise UnsupportedShape(f'selective_scan: {channels} channels of {states} states')
     y = torch.empty((n, channels), dtype=out_dtype, device=u.device)
+    nbytes = lib.qil_selective_scan_workspace(n_seqs, int(max_query), channels, states)
+    workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=u.device) if nbytes else None
     _check(lib.qil_selective_scan(_ptr(u), p_dt, c_dt, s_dt, _ptr(dt_bias), _ptr(a), p_bc, c_bc, s_bc, _ptr(d), p_g, c_g,
                                   s_g, gate_columns, int(gate_offset), _ptr(state), _ptr(cu_seqlens), _ptr(seq_starts),
-                                  _ptr(seq_slots), _ptr(y), _code(out_dtype), n, n_seqs, channels, states, _stream()),
-           'selective_scan')
+                                  _ptr(seq_slots), _ptr(y), _code(out_dtype), n, n_seqs, channels, states, int(max_query),
+                                  _ptr(workspace), _stream()), 'selective_scan')
     return y

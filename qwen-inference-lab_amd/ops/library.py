@@ -332,7 +332,9 @@ def _declare(lib):
     lib.qil_soft_cap.argtypes = [p, f, z, p]
     lib.qil_channel_conv.argtypes = [p, i, i, i, p, p, p, p, p, p, p, p, i, i, i, i, i, p]
     lib.qil_selective_scan_takes.argtypes = [i, i, i]
-    lib.qil_selective_scan.argtypes = [p, p, i, i, p, p, p, i, i, p, p, i, i, i, i, p, p, p, p, p, i, i, i, i, i, p]
+    lib.qil_selective_scan.argtypes = [p, p, i, i, p, p, p, i, i, p, p, i, i, i, i, p, p, p, p, p, i, i, i, i, i, i, p, p]
+    lib.qil_selective_scan_workspace.argtypes = [i, i, i, i]
+    lib.qil_selective_scan_workspace.restype = z
     for name in ('qil_scaled_sum', 'qil_sigmoid_gate', 'qil_soft_cap', 'qil_channel_conv', 'qil_selective_scan_takes',
                  'qil_selective_scan'):
         getattr(lib, name).restype = i

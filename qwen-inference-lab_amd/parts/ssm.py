@@ -68,5 +68,5 @@ class SelectiveScan(Mixer):
         dt = ops.linear(low, p['dt_proj.weight'], None, partials=True)
         bc = ops.linear(u, p['bc_proj.weight'], None, partials=True)
         y = ops.selective_scan(u, dt, bc, xz, dt_bias=p['dt_proj.bias'], a=p['A'], d=p['D'], state=scan_cache.state,
-                               gate_offset=self.inner, out_dtype=self.dtype, **sequences)
+                               gate_offset=self.inner, max_query=ctx.max_query, out_dtype=self.dtype, **sequences)
         return ops.linear(y, p['o_proj.weight'], None, partials=True)

@@ -471,7 +471,7 @@ def channel_conv(x, weight, bias, *, columns, state, cu_seqlens, seq_starts, seq
 
 
 def selective_scan(u, dt, bc, gate, *, dt_bias, a, d, state, gate_offset, cu_seqlens, seq_starts, seq_slots, n_seqs,
-                   out_dtype):
+                   out_dtype, max_query=None):
     n, channels = u.shape
     states = a.shape[1]
     uf, dtf, bcf = u.to(torch.float32), _value(dt).to(torch.float32), _value(bc).to(torch.float32)

@@ -190,8 +190,10 @@ def test_channel_convolution_with_its_state(dtype, channels, taps, splits):
 @pytest.mark.parametrize('channels,states,splits', [(20, 4, 0), (16, 16, 2), (33, 17, 1), (320, 24, 0), (7, 1, 3), (40, 70, 0),
                                                     (24, 130, 1)])
 def test_selective_scan_with_its_state(dtype, channels, states, splits):
-    """Steps over four slots: sequences that begin, continue, bring one row or many; lanes past the last channel and
-    past the last state; inputs as tensors and as partial sums."""
+    """Steps over four slots: sequences that begin, continue, bring one row or many (up to 64 rows of every sequence
+    the step walks each in one piece, beyond that in chunks of 64 tokens side by side, with sequences of one chunk and
+    of a chunk's exact length among them); lanes past the last channel and past the last state, more states than the
+    form with a thread a channel takes; inputs as tensors and as partial sums."""
     if dtype == torch.float32 and splits == 0:
         splits = 1
     g = torch.Generator().manual_seed(channels + states)
@@ -201,7 +203,8 @@ def test_selective_scan_with_its_state(dtype, channels, states, splits):
     state_g = state_c.clone().cuda()
     gate_width, offset = 2 * channels + 5, channels + 2
     steps = [([5, 1], [0, 0], [3, 0]), ([1, 1, 70], [5, 1, 0], [3, 0, 2]), ([2, 130, 1], [6, 0, 70], [3, 1, 2]),
-             ([1, 1, 1, 1], [8, 2, 71, 130], [3, 0, 2, 1]), ([9], [0], [0])]
+             ([1, 1, 1, 1], [8, 2, 71, 130], [3, 0, 2, 1]), ([9], [0], [0]), ([64, 64, 3], [9, 9, 72], [0, 3, 2]),
+             ([65, 300, 128, 1], [73, 73, 75, 131], [0, 3, 2, 1])]
     for counts, starts, slots in steps:
         n = sum(counts)
         u = torch.randn(n, channels, generator=g).to(dtype)
@@ -210,7 +213,7 @@ def test_selective_scan_with_its_state(dtype, channels, states, splits):
         gate = partials(torch.randn(n, gate_width, generator=g).to(dtype), splits, g)
         cu = ints([0] + torch.tensor(counts).cumsum(0).tolist())
         args = dict(cu_seqlens=cu, seq_starts=ints(starts), seq_slots=ints(slots))
-        common = dict(gate_offset=offset, n_seqs=len(counts), out_dtype=dtype)
+        common = dict(gate_offset=offset, n_seqs=len(counts), out_dtype=dtype, max_query=max(counts))
         want = refs.selective_scan(u, host(dt), host(bc), host(gate), dt_bias=dt_bias, a=a, d=d, state=state_c, **args, **common)
         got = ops.selective_scan(u.cuda(), moved(dt), moved(bc), moved(gate), dt_bias=dt_bias.cuda(), a=a.cuda(), d=d.cuda(),
                                  state=state_g, **{k: v.cuda() for k, v in args.items()}, **common)
@@ -237,7 +240,7 @@ def test_a_scan_that_forgets_nothing_adds_up():
         got = ops.selective_scan(u.cuda(), torch.zeros(size, channels).cuda(), torch.ones(size, 2 * states).cuda(),
                                  torch.full((size, channels), 30.0).cuda(), dt_bias=dt_bias.cuda(), a=a.cuda(), d=d.cuda(),
                                  state=state, gate_offset=0, cu_seqlens=ints([0, size]).cuda(), seq_starts=ints([at]).cuda(),
-                                 seq_slots=ints([1]).cuda(), n_seqs=1, out_dtype=torch.float32)
+                                 seq_slots=ints([1]).cuda(), n_seqs=1, max_query=size, out_dtype=torch.float32)
         rows.append(got.cpu())
         at += size
     got = torch.cat(rows)[:, 0]
