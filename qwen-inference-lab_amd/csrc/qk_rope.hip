@@ -32,6 +32,13 @@ __device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t in
   return v;
 }
 
+// The projection's bias (float32, by column of the product; null: none) joins eight summed elements.
+__device__ __forceinline__ void add_bias8(float (&x)[8], const float* __restrict__ bias, int column) {
+  if (!bias) return;
+  const float4 lo = *reinterpret_cast<const float4*>(bias + column), hi = *reinterpret_cast<const float4*>(bias + column + 4);
+  x[0] += lo.x; x[1] += lo.y; x[2] += lo.z; x[3] += lo.w; x[4] += hi.x; x[5] += hi.y; x[6] += hi.z; x[7] += hi.w;
+}
+
 template <typename TD, typename T>
 __global__ void qk_norm_rope_store_kernel(
     const TD* __restrict__ qkv, int splits, size_t split_stride, T* __restrict__ q_out,
@@ -39,7 +46,7 @@ __global__ void qk_norm_rope_store_kernel(
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
     const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
     int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first, int row_elems,
-    float temp_coef, int temp_every) {
+    float temp_coef, int temp_every, const float* __restrict__ bias) {
   __shared__ float vec[QIL_MAX_HEAD_DIM];
   const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const size_t src = (size_t)n * row_elems + (size_t)head * d;    // index into qkv
@@ -55,13 +62,15 @@ __global__ void qk_norm_rope_store_kernel(
       dst = k_cache + ((page * kv_heads + kvh) * page_size + offset) * d;
     } else {                                             // v: copy, transposed within the page
       T* column = v_cache + (page * kv_heads + kvh) * (size_t)d * page_size + offset;
-      for (int i = lane; i < d; i += QIL_WAVE) st(column + (size_t)i * page_size, load_sum(qkv, src + i, splits, split_stride));
+      for (int i = lane; i < d; i += QIL_WAVE)
+        st(column + (size_t)i * page_size, load_sum(qkv, src + i, splits, split_stride) + (bias ? bias[head * d + i] : 0.f));
       return;
     }
   }
 
   const float* weight = is_q ? q_weight : k_weight;
-  for (int i = lane; i < d; i += QIL_WAVE) vec[i] = load_sum(qkv, src + i, splits, split_stride);
+  for (int i = lane; i < d; i += QIL_WAVE)
+    vec[i] = load_sum(qkv, src + i, splits, split_stride) + (bias ? bias[head * d + i] : 0.f);
   __syncthreads();
   const int half = rot / 2;
   const int position = positions[n];
@@ -117,7 +126,7 @@ qk_norm_rope_store_vec_kernel(
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size,
     float eps, int tg_log2, unsigned v_first_block, int norm_dim, int rotate_first, int row_elems, float temp_coef,
-    int temp_every) {
+    int temp_every, const float* __restrict__ bias) {
   const int total_heads = heads + 2 * kv_heads;
   const int TG = 1 << tg_log2;
   if (blockIdx.x >= v_first_block) {
@@ -134,6 +143,7 @@ qk_norm_rope_store_vec_kernel(
     if (token >= (size_t)n) return;
     float x[8];
     load8_sum(qkv, token * row_elems + (size_t)(heads + kv_heads + kvh) * d + chunk * 8, splits, split_stride, x);
+    add_bias8(x, bias, (heads + kv_heads + kvh) * d + chunk * 8);
     const int slot = slots[token];
     const size_t page = slot / page_size, offset = slot % page_size;
     T* column = v_cache + ((page * kv_heads + kvh) * (size_t)d + chunk * 8) * page_size + offset;
@@ -150,6 +160,7 @@ qk_norm_rope_store_vec_kernel(
   if (!is_q && slots == nullptr) return;
   float x[8];
   load8_sum(qkv, (size_t)token * row_elems + (size_t)head * d + chunk * 8, splits, split_stride, x);
+  add_bias8(x, bias, head * d + chunk * 8);
 
   if (!is_q && !is_k) {                                 // v: copy, transposed within the page
     const int kvh = head - heads - kv_heads, slot = slots[token];
@@ -182,12 +193,14 @@ qk_norm_rope_store_vec_kernel(
 // than d when the heads are padded with zeros to a size the attention kernels take.
 // extra_columns: so many more columns follow the v heads in every row of qkv (another branch's part of a stacked
 // product); they are skipped.  kv_heads 0: the rows hold queries only (a reader of another entry's cache).
+// bias: null, or float32 [(heads + 2 kv_heads) d]: the projection's bias, added to the sums as they are loaded (the
+// product before this kernel then needs none, and may leave partial sums).
 // temp_every > 0: the query at position p is multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) last.
 extern "C" int qil_qk_norm_rope_store(
     const void* qkv, int in_dtype, int splits, void* q_out, const float* q_weight, const float* k_weight,
     const float* cos_table, const float* sin_table, const int* positions, const int* slots, void* k_cache,
     void* v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first,
-    int extra_columns, float temp_coef, int temp_every, int dtype, hipStream_t s) {
+    int extra_columns, float temp_coef, int temp_every, const float* bias, int dtype, hipStream_t s) {
   if (n == 0) return 0;
   if (extra_columns < 0 || temp_every < 0 || kv_heads < 0 || (kv_heads == 0 && slots)) return -1;
   const int row_elems = (heads + 2 * kv_heads) * d + extra_columns;
@@ -205,7 +218,7 @@ extern "C" int qil_qk_norm_rope_store(
   const bool rot_fits = rot == 0 || !cos_table || (rot % 16 == 0 && (half_chunks & (half_chunks - 1)) == 0);
   const bool aligned = row_elems % 8 == 0 &&
                        (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)q_weight | (uintptr_t)k_weight |
-                         (uintptr_t)cos_table | (uintptr_t)sin_table) % 16) == 0;
+                         (uintptr_t)cos_table | (uintptr_t)sin_table | (uintptr_t)bias) % 16) == 0;
   if (tg_log2 > 0 && rot_fits && aligned) {
     // v in blocks of its own behind the others when a head has at least four chunks and there is a cache to write
     const bool v_apart = tg_log2 >= 2 && slots != nullptr;
@@ -218,7 +231,7 @@ extern "C" int qil_qk_norm_rope_store(
   hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)qkv, splits,    \
                      stride, (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache,       \
                      (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block, norm_dim, rotate_first,       \
-                     row_elems, temp_coef, temp_every)
+                     row_elems, temp_coef, temp_every, bias)
     if (dtype == QIL_F32) QIL_QKV_CASE(float, float);
     else if (in_dtype == QIL_F32) QIL_QKV_CASE(float, bf16_t);
     else QIL_QKV_CASE(bf16_t, bf16_t);
@@ -228,7 +241,7 @@ extern "C" int qil_qk_norm_rope_store(
 #define QIL_QK_CASE(TD, T)                                                                                            \
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TD, T>), grid, dim3(QIL_WAVE), 0, s, (const TD*)qkv, splits, stride,   \
                      (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache, (T*)v_cache,  \
-                     heads, kv_heads, d, rot, page_size, eps, norm_dim, rotate_first, row_elems, temp_coef, temp_every)
+                     heads, kv_heads, d, rot, page_size, eps, norm_dim, rotate_first, row_elems, temp_coef, temp_every, bias)
   if (dtype == QIL_F32) QIL_QK_CASE(float, float);
   else if (in_dtype == QIL_F32) QIL_QK_CASE(float, bf16_t);
   else QIL_QK_CASE(bf16_t, bf16_t);

@@ -71,6 +71,87 @@ __global__ void channel_conv_kernel(Operand x, int x_columns, const float* __res
   }
 }
 
+
+// The same with V neighbouring channels a thread (V = 8 for a bfloat16 input, 4 for float32 partial sums: 16-byte
+// loads of the input, the factors and the state), for sizes and addresses that allow it.
+template <typename TI, int V> struct conv_in;
+template <> struct conv_in<bf16_t, 8> {
+  static __device__ __forceinline__ void load(const bf16_t* base, size_t index, int, size_t, float* out) { ld8(base + index, out); }
+};
+template <> struct conv_in<float, 4> {
+  static __device__ __forceinline__ void load(const float* base, size_t index, int splits, size_t stride, float* out) {
+    float4 v = ld4(base + index);
+    for (int s = 1; s < splits; ++s) {
+      const float4 w = ld4(base + (size_t)s * stride + index);
+      v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+    }
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  }
+};
+template <int V> __device__ __forceinline__ void load_floats(const float* p, float* out) {
+#pragma unroll
+  for (int e = 0; e < V; e += 4) { const float4 v = ld4(p + e); out[e] = v.x; out[e + 1] = v.y; out[e + 2] = v.z; out[e + 3] = v.w; }
+}
+template <int V> __device__ __forceinline__ void store_floats(float* p, const float* v) {
+#pragma unroll
+  for (int e = 0; e < V; e += 4) st4(p + e, make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]));
+}
+template <int V> __device__ __forceinline__ void store_floats(bf16_t* p, const float* v) {
+#pragma unroll
+  for (int e = 0; e < V; e += 4) st4(p + e, make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]));
+}
+
+template <typename TI, typename T, int V>
+__global__ void channel_conv_vec_kernel(const TI* __restrict__ x, int splits, size_t split_stride, int x_columns,
+                                        const float* __restrict__ w, const float* __restrict__ bias, float* state,
+                                        const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts,
+                                        const int* __restrict__ seq_slots, const int* __restrict__ row_seq,
+                                        T* __restrict__ out, int channels, int taps, int act) {
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * V, n = blockIdx.x;
+  if (c >= channels) return;
+  const int keep = taps - 1;
+  const int s = row_seq[n], row0 = cu_seqlens[s], t = n - row0;
+  if (t > 0 && t < keep) return;                       // computed with the sequence's first row
+  const int rows = cu_seqlens[s + 1] - row0, start = seq_starts[s];
+  float* held = state ? state + (size_t)seq_slots[s] * keep * channels : nullptr;
+  const int upto = t == 0 ? min(rows, max(keep, 1)) : t + 1;
+  float b[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) b[e] = 0.f;
+  if (bias) load_floats<V>(bias + c, b);
+  for (int r = t; r < upto; ++r) {
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = b[e];
+    for (int j = 0; j < taps; ++j) {
+      const int source = r - keep + j;
+      float in[V], f[V];
+      if (source >= 0) conv_in<TI, V>::load(x, (size_t)(row0 + source) * x_columns + c, splits, split_stride, in);
+      else if (held && start + source >= 0) load_floats<V>(held + (size_t)(keep + source) * channels + c, in);
+      else continue;
+      load_floats<V>(w + (size_t)j * channels + c, f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += f[e] * in[e];
+    }
+    if (act) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = silu_f(acc[e]);
+    }
+    store_floats<V>(out + (size_t)(row0 + r) * channels + c, acc);
+  }
+  if (t == 0 && held) {
+    for (int k = 0; k < keep; ++k) {
+      const int source = rows - keep + k;
+      float in[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) in[e] = 0.f;
+      if (source >= 0) conv_in<TI, V>::load(x, (size_t)(row0 + source) * x_columns + c, splits, split_stride, in);
+      else if (start + source >= 0) load_floats<V>(held + (size_t)(k + rows) * channels + c, in);
+      store_floats<V>(held + (size_t)k * channels + c, in);
+    }
+  }
+}
+
 __device__ __forceinline__ float row16_total(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
@@ -161,7 +242,13 @@ template <bool FAST> __device__ __forceinline__ float scan_silu(float v) {
 // PHASE 0: a sequence's rows from its stored state, y and the new state written.  PHASE 1: a chunk from zero; its end
 // state goes to carry[seq * max_chunks + chunk][channel][NS] and its sum of steps to sums[..][channel].  PHASE 2: a
 // chunk from the state that the carry kernel left in carry[..]; y written.
-template <typename T, int NS, int PHASE>
+// DIRECT: dt_raw, bc and gate are plain arrays of T (what the products of many rows leave): typed loads, no branches.
+template <bool DIRECT, typename T> __device__ __forceinline__ float scan_fetch(const Operand& x, size_t index) {
+  if (DIRECT) return ld(reinterpret_cast<const T*>(x.data) + index);
+  return operand_at(x, index);
+}
+
+template <typename T, int NS, int PHASE, bool DIRECT>
 __global__ void __launch_bounds__(SCAN_THREADS)
 scan_chunk_kernel(const T* __restrict__ u, Operand dt_raw, const float* __restrict__ dt_bias,
                   const float* __restrict__ a, Operand bc, const float* __restrict__ d, Operand gate, int gate_columns,
@@ -203,7 +290,7 @@ scan_chunk_kernel(const T* __restrict__ u, Operand dt_raw, const float* __restri
     __syncthreads();                                   // the tile before this one has been used
     for (int i = threadIdx.x; i < rows * 2 * NS; i += SCAN_THREADS) {
       const int r = i / (2 * NS), k = i - r * 2 * NS, half = k / NS, n = k - half * NS;
-      tile[i] = n < states ? operand_at(bc, (size_t)(t0 + r) * 2 * states + half * states + n) : 0.f;
+      tile[i] = n < states ? scan_fetch<DIRECT, T>(bc, (size_t)(t0 + r) * 2 * states + half * states + n) : 0.f;
     }
     __syncthreads();
     for (int r0 = 0; r0 < rows; r0 += 8) {
@@ -211,9 +298,9 @@ scan_chunk_kernel(const T* __restrict__ u, Operand dt_raw, const float* __restri
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const size_t t = min(t0 + r0 + k, last - 1);
-        dt[k] = operand_at(dt_raw, t * channels + cc);
+        dt[k] = scan_fetch<DIRECT, T>(dt_raw, t * channels + cc);
         uv[k] = ld(u + t * channels + cc);
-        zv[k] = PHASE == 1 ? 0.f : operand_at(gate, t * gate_columns + gate_offset + cc);
+        zv[k] = PHASE == 1 ? 0.f : scan_fetch<DIRECT, T>(gate, t * gate_columns + gate_offset + cc);
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
@@ -282,6 +369,25 @@ int qil_channel_conv(const void* x, int x_code, int x_splits, int x_columns, con
   if (n == 0) return 0;
   if (channels < 1 || channels > x_columns || taps < 1 || (taps > 1 && !state) || x_splits < 1 ||
       (x_code == QIL_BF16 && x_splits != 1)) return -1;
+  const int V = x_code == QIL_BF16 ? 8 : 4;
+  if (channels % V == 0 && x_columns % V == 0 &&
+      (((uintptr_t)x | (uintptr_t)w | (uintptr_t)bias | (uintptr_t)state | (uintptr_t)out) % 16) == 0 &&
+      !(x_code == QIL_BF16 && out_dtype == QIL_F32)) {
+    const int lanes = channels / V;
+    const int threads = lanes >= 128 ? 128 : (lanes + 63) / 64 * 64;
+    const dim3 grid(n, (lanes + threads - 1) / threads);
+    const size_t stride = (size_t)n * x_columns;
+    if (x_code == QIL_BF16)
+      hipLaunchKernelGGL((channel_conv_vec_kernel<bf16_t, bf16_t, 8>), grid, dim3(threads), 0, s, (const bf16_t*)x, 1, stride,
+                         x_columns, w, bias, state, cu_seqlens, seq_starts, seq_slots, row_seq, (bf16_t*)out, channels, taps, act);
+    else if (out_dtype == QIL_F32)
+      hipLaunchKernelGGL((channel_conv_vec_kernel<float, float, 4>), grid, dim3(threads), 0, s, (const float*)x, x_splits, stride,
+                         x_columns, w, bias, state, cu_seqlens, seq_starts, seq_slots, row_seq, (float*)out, channels, taps, act);
+    else
+      hipLaunchKernelGGL((channel_conv_vec_kernel<float, bf16_t, 4>), grid, dim3(threads), 0, s, (const float*)x, x_splits, stride,
+                         x_columns, w, bias, state, cu_seqlens, seq_starts, seq_slots, row_seq, (bf16_t*)out, channels, taps, act);
+    QIL_RETURN_LAUNCH_STATUS();
+  }
   const Operand in{x, x_code, x_splits, (size_t)n * x_columns};
   const int threads = channels >= 256 ? 256 : (channels + 63) / 64 * 64;
   const dim3 grid(n, (channels + threads - 1) / threads);
@@ -323,10 +429,14 @@ int qil_selective_scan(const void* u, const void* dt_raw, int dt_code, int dt_sp
     float* carry = workspace;
     const int ns = (states + 7) / 8 * 8;
     float* sums = workspace ? workspace + (size_t)n_seqs * chunks * channels * ns : nullptr;
+    const bool direct = dt_code == dtype && bc_code == dtype && gate_code == dtype && dt_splits == 1 && bc_splits == 1 &&
+                        gate_splits == 1;
+#define QIL_CHUNK_D(T, NS, PHASE, DIRECT)                                                                             \
+  hipLaunchKernelGGL((scan_chunk_kernel<T, NS, PHASE, DIRECT>), blocks, dim3(SCAN_THREADS), 0, s, (const T*)u, odt,    \
+                     dt_bias, a, obc, d, og, gate_columns, gate_offset, state, cu_seqlens, seq_starts, seq_slots, (T*)y, \
+                     channels, states, carry, sums, chunks)
 #define QIL_CHUNK(T, NS, PHASE)                                                                                       \
-  hipLaunchKernelGGL((scan_chunk_kernel<T, NS, PHASE>), blocks, dim3(SCAN_THREADS), 0, s, (const T*)u, odt, dt_bias, a, \
-                     obc, d, og, gate_columns, gate_offset, state, cu_seqlens, seq_starts, seq_slots, (T*)y, channels,  \
-                     states, carry, sums, chunks)
+  do { if (direct) QIL_CHUNK_D(T, NS, PHASE, true); else QIL_CHUNK_D(T, NS, PHASE, false); } while (0)
 #define QIL_CHUNK_NS(T, PHASE)                                                                                        \
   do {                                                                                                                \
     if (ns == 8) QIL_CHUNK(T, 8, PHASE); else if (ns == 16) QIL_CHUNK(T, 16, PHASE);                                   \
@@ -346,6 +456,7 @@ int qil_selective_scan(const void* u, const void* dt_raw, int dt_code, int dt_sp
 #undef QIL_CHUNK_T
 #undef QIL_CHUNK_NS
 #undef QIL_CHUNK
+#undef QIL_CHUNK_D
     QIL_RETURN_LAUNCH_STATUS();
   }
   const dim3 grid((channels + 15) / 16, n_seqs);

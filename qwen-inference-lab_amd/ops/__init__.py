@@ -581,7 +581,7 @@ def _rotation_arguments(rotation, head_dim):
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
                        k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False, extra_columns=0,
-                       q_temperature=None):
+                       q_temperature=None, bias=None):
     """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given).  ``norm_dim``: the
     number of elements the norm's mean runs over when the heads are padded with zeros (default: head_dim).
     ``rotate_first``: the rotation comes before the norm.  A rotation that carries ``frequencies`` is applied from
@@ -589,13 +589,17 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
     ``extra_columns``: so many more columns follow the v heads in every row of ``qkv`` (another branch of a stacked
     product); they are skipped.  ``kv_heads`` 0: the rows hold queries only.  ``q_temperature`` (coef, every): the
-    query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) last, in float32.
+    query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) last, in float32.  ``bias``
+    float32 [(heads + 2 kv_heads) d]: the projection's bias, added here (the product before then has none and may
+    stay partial sums).
 
     ``qkv`` [N, (heads + 2 kv_heads) d + extra_columns]: tensor of type ``dtype`` or Partials.  Returns q as ``dtype``
     [N, heads * d]; k and v go into the caches at ``slots`` (None: not stored)."""
     n = qkv.shape[0]
     pointer, code, splits = _operand(qkv, 'qkv', dtype, (n, (heads + 2 * kv_heads) * head_dim + extra_columns))
     coef, every = q_temperature if q_temperature is not None else (0.0, 0)
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, ((heads + 2 * kv_heads) * head_dim,))
     _require(positions, 'positions', torch.int32, (n,))
     for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
         if w is not None:
@@ -610,7 +614,8 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
     _check(library.load().qil_qk_norm_rope_store(
         pointer, code, splits, _ptr(q), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions),
         _ptr(slots), _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps),
-        int(norm_dim or 0), int(bool(rotate_first)), int(extra_columns), float(coef), int(every), _code(dtype), _stream()),
+        int(norm_dim or 0), int(bool(rotate_first)), int(extra_columns), float(coef), int(every), _ptr(bias), _code(dtype),
+        _stream()),
         'qk_norm_rope_store')
     return q
 

@@ -128,6 +128,8 @@ class Attention(Mixer):
                 biases.append(biases[0].new_zeros(self.heads * self.padded_dim))
         self.w_qkv = torch.cat(matrices).contiguous()
         self.b_qkv = torch.cat(biases).contiguous() if self.bias else None
+        # the bias of q, k and v alone (the gate has none), as the q/k kernel takes it
+        self.b_qkv_own = torch.cat(biases[:len(stacked)]).contiguous() if self.bias else None
         p['qkv_proj.weight'] = self.w_qkv
         if self.bias:
             p['qkv_proj.bias'] = self.b_qkv
@@ -146,7 +148,9 @@ class Attention(Mixer):
         p = self.p
         if cache.writes and not self.own_kv:
             raise ValueError('an attention part without keys and values of its own reads another entry\'s cache')
-        qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
+        extended = self.gate or self.sink or self.q_temperature is not None or not self.own_kv
+        # (the extended step's q/k kernel adds the bias itself: its product may then stay partial sums)
+        qkv = ops.linear(h, self.w_qkv, None if extended else self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
         if self.qk_norm_eps is not None and not self.qk_norm_weights:
             norms = dict(q_weight=self._ones, k_weight=self._ones, eps=self.qk_norm_eps)
@@ -154,7 +158,7 @@ class Attention(Mixer):
             norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight', p.get('q_norm.weight')),
                          eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
         sizes = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.padded_dim)
-        if self.gate or self.sink or self.q_temperature is not None or not self.own_kv:
+        if extended:
             return self._forward_extended(qkv, rotation, norms, sizes, ctx, cache)
         # (the kernel that makes its queries itself norms over the whole head it sees: not for padded heads)
         if ctx.max_query == 1 and self.padded_dim == self.head_dim and \
@@ -189,7 +193,7 @@ class Attention(Mixer):
             qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,
             k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype, norm_dim=self.head_dim,
             rotate_first=self.norm_after_rotation, heads=self.heads, kv_heads=stored, head_dim=self.padded_dim,
-            extra_columns=gate_columns, q_temperature=self.q_temperature, **norms)
+            extra_columns=gate_columns, q_temperature=self.q_temperature, bias=self.b_qkv_own, **norms)
         attended = ops.paged_attention(
             q, k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,

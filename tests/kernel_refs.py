@@ -84,10 +84,13 @@ def silu_mul(gate_up, out_dtype=None, interleaved=False):
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
                        k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False, extra_columns=0,
-                       q_temperature=None):
+                       q_temperature=None, bias=None):
     qkv = _value(qkv)
     n, d = qkv.shape[0], head_dim
-    x = qkv[:, :(heads + 2 * kv_heads) * d].reshape(n, heads + 2 * kv_heads, d)
+    x = qkv[:, :(heads + 2 * kv_heads) * d]
+    if bias is not None:
+        x = x.to(torch.float32) + bias
+    x = x.reshape(n, heads + 2 * kv_heads, d)
     q, k, v = x[:, :heads].to(torch.float32), x[:, heads:heads + kv_heads].to(torch.float32), x[:, heads + kv_heads:]
 
     def normed(t, weight):

@@ -59,6 +59,9 @@ def host(x):
     ([129, 64, 1000, 16], [129, 1, 3, 16], 16, 128, 8, 2, None),
     ([257, 100], [200, 31], 3, 40, 6, 2, 64),
     ([513], [513], 16, 64, 4, 2, 100),
+    ([1200], [1200], 16, 128, 4, 2, 300),                       # the bfloat16 kernel for heads of 128, a long prompt
+    ([1500, 900], [700, 900], 16, 128, 8, 8, None),
+    ([1100], [1100], 16, 64, 4, 1, 512),
 ])
 def test_attention_with_sinks(dtype, lengths, chunks, page_size, d, heads, kv_heads, window, monkeypatch):
     """One more term exp(sink) in every head's divisor, sinks from far below to far above the scores; with the keys in
@@ -112,17 +115,18 @@ def test_queries_with_a_temperature_and_columns_to_skip(dtype, heads, kv_heads, 
         from qil_amd.parts import RotaryFrequencies
         rotation = RotaryFrequencies(rot, 300.0, scaling=(4.0, 1.0, 4.0, 64)).rotation()
     caches = [torch.zeros(pages, max(kv_heads, 1), page_size, d).to(dtype), torch.zeros(pages, max(kv_heads, 1), d, page_size).to(dtype)]
+    bias = torch.randn((heads + 2 * kv_heads) * d, generator=g)
     args = dict(heads=heads, kv_heads=kv_heads, head_dim=d, eps=1e-5, page_size=page_size, dtype=dtype, extra_columns=extra,
                 q_temperature=(0.6, 7))
     kc, vc = caches[0].clone(), caches[1].clone()
     want = refs.qk_norm_rope_store(host(qkv), q_weight=ones, k_weight=ones, rotation=rotation, positions=positions,
-                                   slots=slots if kv_heads else None, k_cache=kc, v_cache=vc, **args)
+                                   slots=slots if kv_heads else None, k_cache=kc, v_cache=vc, bias=bias, **args)
     gk, gv = caches[0].cuda(), caches[1].cuda()
     if rotation is not None:
         rotation = type(rotation)(None, None, rotation.rot_dim, rotation.frequencies.cuda())
     got = ops.qk_norm_rope_store(moved(qkv), q_weight=ones.cuda(), k_weight=ones.cuda(), rotation=rotation,
                                  positions=positions.cuda(), slots=slots.cuda() if kv_heads else None, k_cache=gk, v_cache=gv,
-                                 **args)
+                                 bias=bias.cuda(), **args)
     close(got, want, dtype, 3.0)
     plain_args = dict(args, q_temperature=None)
     cold = refs.qk_norm_rope_store(host(qkv), q_weight=ones, k_weight=ones, rotation=None, positions=positions, slots=None,
@@ -153,7 +157,8 @@ def test_gate_sum_and_cap(dtype, splits):
 
 # ------------------------------------------------------------------------------------------------ channel convolution
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('channels,taps,splits', [(20, 4, 0), (21, 1, 2), (7, 2, 1), (320, 4, 0), (300, 3, 3), (1028, 6, 0)])
+@pytest.mark.parametrize('channels,taps,splits', [(20, 4, 0), (21, 1, 2), (7, 2, 1), (320, 4, 0), (300, 3, 3), (1028, 6, 0),
+                                                  (64, 4, 2), (1024, 2, 0), (8, 5, 1)])
 def test_channel_convolution_with_its_state(dtype, channels, taps, splits):
     """Steps over five slots: sequences that begin (whatever their slot held before, NaN here, is not read), that
     continue from a state shorter than taps - 1 inputs, that bring fewer rows than the state holds, and one long
@@ -161,7 +166,7 @@ def test_channel_convolution_with_its_state(dtype, channels, taps, splits):
     if dtype == torch.float32 and splits == 0:
         splits = 1
     g = torch.Generator().manual_seed(channels * 10 + taps)
-    keep, width = taps - 1, 2 * channels + 3
+    keep, width = taps - 1, 2 * channels + (3 if channels % 4 else 8)
     weight, bias = torch.randn(taps, channels, generator=g), torch.randn(channels, generator=g)
     state_c = torch.full((5, keep, channels), float('nan')) if keep else None
     state_g = state_c.clone().cuda() if keep else None
