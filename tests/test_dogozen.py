@@ -192,6 +192,25 @@ def test_decoding_token_by_token_equals_the_prompt(case):
     case.close(feed(runner, 'r', tokens, [50]), case.expected(tokens), '50, then 90 single tokens')
 
 
+@pytest.mark.parametrize('name', sorted(CONFIGS))
+def test_a_long_prompt(name, backend, tmp_path):
+    """Several hundred tokens at once (the scan in chunks side by side, the attention's keys in many tiles), then two
+    long portions and single tokens; the late places are compared.  The routed feed-forwards are made dense here: among
+    hundreds of tokens some router's choice is a close call, and every later place would have to be left out."""
+    config, seed, page_size, spread = CONFIGS[name]
+    config = json.loads(json.dumps(config))
+    for layer in config['layers']:
+        if layer['mlp'] is not None and layer['mlp']['kind'] == 'moe':
+            layer['mlp'] = plain.dense_mlp(layer['mlp']['expert']['ff'] + 8)
+    case = make_case(name, config, plain.random_weights(config, seed, spread), backend, tmp_path / name, page_size)
+    runner = case.runner(pages=-(-700 // case.page_size) + 2)
+    tokens = tokens_for(case.config, 650, 10)
+    late = list(range(560, 650))
+    expected = case.expected(tokens)[late]
+    case.close(feed(runner, 'r', tokens, [650], late), expected, 'whole')
+    case.close(feed(runner, 'r', tokens, [130, 470, 3], late), expected, 'two long portions, then single tokens')
+
+
 def test_decode_graphs_replay_the_same_logits(case):
     if case.model.device.type != 'cuda':
         pytest.skip('graphs are a GPU matter')
@@ -557,6 +576,18 @@ def test_config_round_trip_and_refusals():
                    dict(config, layers=[dict(layers[1], mlp=dict(kind='dense', ff=8, limit=1.0))])):
         with pytest.raises(ConfigError):
             DogozenConfig.from_dict(broken)
+
+
+def test_the_bench_makes_valid_configurations():
+    """The configurations that ``bench.py --phase designs --design dogozen`` measures are ones the design accepts."""
+    import bench
+    from qil_amd.config import DogozenConfig
+    sizes = dict(width=64, ff=96, heads=4, dim=16, rot_dim=8)
+    for kind in ('turns', 'attention', 'attention-routed', 'parallel', 'window'):
+        typed = DogozenConfig.from_dict(bench.dogozen_config(sizes, 6, 100, 32, kind))
+        assert len(typed.layers) == 6
+    assert typed.layers[0]['type'] == 'parallel'
+    assert bench.dogozen_config(sizes, 6, 100, 32, 'turns')['layers'][3]['mixer']['kv_from'] == 1
 
 
 def test_optional_keys_may_be_absent(tmp_path, cpu_kernels):
