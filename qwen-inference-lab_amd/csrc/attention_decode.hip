@@ -44,6 +44,11 @@ struct FusedQKV {
   int rot;
   int rotate_first;                                        // the rotation comes before the head norm
   int writes;                                              // 0: the cache belongs to another layer, which wrote it
+  int row_elems;                                           // elements of a row of qkv (more than q, k and v where another
+                                                           // branch's columns follow; q alone for a reader without k and v)
+  const float* bias;                                       // null, or the projection's bias by column, added to the sums
+  float temp_coef;                                         // temp_every > 0: the query at position p is multiplied by
+  int temp_every;                                          // 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) last
 };
 
 // Keys and values are read once a step by one block (the whole group of query heads is served by it).
@@ -227,27 +232,34 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
   auto make_queries = [&]() {
     if constexpr (FUSED) {
       constexpr int TG = DMAX / 8, HPP = QIL_WAVE / TG;      // lanes of a head (8 elements each), heads a pass
-      const int total_heads = heads + 2 * kv_heads;
       const int chunk = lane % TG, sub = lane / TG;
       // the block's waves share the heads (HPP of them a wave and pass); the queries meet in LDS
       uint4* shared_q = reinterpret_cast<uint4*>(lds);       // [g][TG] chunks; the end of the kernel uses the LDS again
       for (int base = wave * HPP; base < g; base += waves * HPP) {
         float x[8];
         const int head = kvh * g + min(base + sub, g - 1);   // lanes past the group repeat its last head
-        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + head) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        load8_sum_wide(fused.qkv, (size_t)row * fused.row_elems + (size_t)head * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        add_bias8(x, fused.bias, head * DMAX + chunk * 8);
         norm_rope8<bf16_t>(x, chunk, TG, fused.q_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot,
                            fused.rotate_first != 0);
+        if (fused.temp_every > 0) {
+          const float temperature = query_temperature(pos, fused.temp_coef, fused.temp_every);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] *= temperature;
+        }
         if (base + sub < g) shared_q[(base + sub) * TG + chunk] = pack8(x);
       }
       owner = fused.writes && pos >= begin && pos < end && wave == ((pos >> 5) - first_step) % waves;
       if (owner) {                                           // wave-uniform
         float x[8];
-        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kvh) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        load8_sum_wide(fused.qkv, (size_t)row * fused.row_elems + (size_t)(heads + kvh) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
+        add_bias8(x, fused.bias, (heads + kvh) * DMAX + chunk * 8);
         norm_rope8<bf16_t>(x, chunk, TG, fused.k_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot,
                            fused.rotate_first != 0);
         new_k = pack8(x);
-        load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kv_heads + kvh) * DMAX + chunk * 8, fused.splits,
+        load8_sum_wide(fused.qkv, (size_t)row * fused.row_elems + (size_t)(heads + kv_heads + kvh) * DMAX + chunk * 8, fused.splits,
                        fused.split_stride, x);
+        add_bias8(x, fused.bias, (heads + kv_heads + kvh) * DMAX + chunk * 8);
         new_v = pack8(x);
         if (sub == 0) {                                      // into the pages (qil/cache.py:79-82)
           const size_t page = table[pos / page_size];
@@ -418,15 +430,19 @@ extern "C" int qil_attn_decode_fused_takes(int heads, int kv_heads, int d, int p
 // rows are the step's rows 0 .. rows-1 (no row index).  q_weight, k_weight: both or neither; cos/sin: both
 // [positions][rot / 2], or neither, or a cos_table alone that holds the rot / 2 frequencies (the angles are then made
 // in the kernel).  rotate_first: rotate, then norm.  softcap > 0: scores are capped softly after the scale.  writes != 0: the new keys and values go into the caches at the rows'
-// positions (the page comes from the block table).
+// positions (the page comes from the block table).  has_kv 0: the rows of qkv hold queries only (a reader; writes must be 0).
+// extra_columns: so many more columns follow in every row and are skipped.  bias: null, or float32 by column of q, k and v.
+// temp_every > 0: the query temperature of qk_rope.hip.  sinks: null, or float32 [heads] (as in qil_attn_decode).
 extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* q_weight, const float* k_weight,
                                      float eps, const float* cos_table, const float* sin_table, int rot, int writes,
                                      void* k_cache, void* v_cache, const int* block_tables, int table_stride,
                                      const int* row_seq, const int* positions, void* workspace, void* out, int rows,
                                      int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
                                      int parts, int waves, int pairs, int rotate_first, float softcap,
-                                     hipStream_t s) {
+                                     int has_kv, int extra_columns, const float* bias, float temp_coef, int temp_every,
+                                     const float* sinks, hipStream_t s) {
   if (rows == 0) return 0;
+  if (extra_columns < 0 || temp_every < 0 || (writes && !has_kv) || ((uintptr_t)bias % 16) || extra_columns % 8) return -1;
   if (!qil_attn_decode_fused_takes(heads, kv_heads, d, page_size, cos_table ? rot : 0) || P % 32 || P < 32 ||
       parts < 1 || parts > 65535 || kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES || splits < 1 ||
       (q_weight == nullptr) != (k_weight == nullptr) || (sin_table != nullptr && cos_table == nullptr) ||
@@ -441,7 +457,9 @@ extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* 
   dim3 grid(rows, kv_heads, parts);
   FusedQKV fused;
   fused.qkv = qkv;
-  fused.split_stride = (size_t)rows * (heads + 2 * kv_heads) * d;
+  fused.row_elems = (heads + (has_kv ? 2 * kv_heads : 0)) * d + extra_columns;
+  fused.split_stride = (size_t)rows * fused.row_elems;
+  fused.bias = bias; fused.temp_coef = temp_coef; fused.temp_every = temp_every;
   fused.splits = splits;
   fused.q_weight = q_weight; fused.k_weight = k_weight; fused.eps = eps;
   fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rot = cos_table ? rot : 0;
@@ -450,7 +468,6 @@ extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* 
   const void* q = nullptr;
   const int q_stride = 0;
   const int* row_index = nullptr;
-  const float* sinks = nullptr;
 #define QIL_DEC_CASE(DMAX)                                                                                          \
   if (pairs) QIL_DEC_LAUNCH(DMAX, true, true, fused);                                                               \
   else QIL_DEC_LAUNCH(DMAX, false, true, fused)

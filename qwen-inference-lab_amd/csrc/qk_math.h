@@ -11,6 +11,13 @@ __device__ __forceinline__ float query_temperature(int position, float coef, int
   return every > 0 ? 1.f + coef * logf((float)((position + 1) / every) + 1.f) : 1.f;
 }
 
+// The projection's bias (float32, by column of the product; null: none) joins eight summed elements.
+__device__ __forceinline__ void add_bias8(float (&x)[8], const float* __restrict__ bias, int column) {
+  if (!bias) return;
+  const float4 lo = *reinterpret_cast<const float4*>(bias + column), hi = *reinterpret_cast<const float4*>(bias + column + 4);
+  x[0] += lo.x; x[1] += lo.y; x[2] += lo.z; x[3] += lo.w; x[4] += hi.x; x[5] += hi.y; x[6] += hi.z; x[7] += hi.w;
+}
+
 __device__ __forceinline__ void load8_sum(const float* base, size_t index, int splits, size_t stride, float* out) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) out[e] = 0.f;

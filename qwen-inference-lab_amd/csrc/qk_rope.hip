@@ -32,13 +32,6 @@ __device__ __forceinline__ float load_sum(const TD* __restrict__ base, size_t in
   return v;
 }
 
-// The projection's bias (float32, by column of the product; null: none) joins eight summed elements.
-__device__ __forceinline__ void add_bias8(float (&x)[8], const float* __restrict__ bias, int column) {
-  if (!bias) return;
-  const float4 lo = *reinterpret_cast<const float4*>(bias + column), hi = *reinterpret_cast<const float4*>(bias + column + 4);
-  x[0] += lo.x; x[1] += lo.y; x[2] += lo.z; x[3] += lo.w; x[4] += hi.x; x[5] += hi.y; x[6] += hi.z; x[7] += hi.w;
-}
-
 template <typename TD, typename T>
 __global__ void qk_norm_rope_store_kernel(
     const TD* __restrict__ qkv, int splits, size_t split_stride, T* __restrict__ q_out,

@@ -670,15 +670,26 @@ def decode_attention_takes(qkv, *, heads, kv_heads, head_dim, page_size, rotatio
 
 def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, writes, k_cache,
                      v_cache, page_size, block_tables, row_seq, max_context, scale, window, unmerged=False,
-                     rotate_first=False, softcap=None):
+                     rotate_first=False, softcap=None, has_kv=True, extra_columns=0, bias=None, q_temperature=None, sinks=None):
     """``qk_norm_rope_store`` and ``paged_attention`` in one kernel for a step whose rows are all alone in their
     sequences: queries, the new key and the new value are made from the partial sums ``qkv`` inside the
     attention kernel (bit for bit what the two kernels make), the new key and value are written into the
     pages (``writes``) and used from registers.  ``rotate_first`` and ``softcap`` as in ``qk_norm_rope_store`` and
-    ``paged_attention``.  Returns what ``paged_attention`` returns."""
+    ``paged_attention``.  ``has_kv=False`` (with ``writes`` False): the rows of ``qkv`` hold queries only;
+    ``extra_columns``, ``bias``, ``q_temperature`` as in ``qk_norm_rope_store``, ``sinks`` as in ``paged_attention``
+    (a step with sinks comes back merged).  Returns what ``paged_attention`` returns."""
     n = qkv.shape[0]
     dtype = torch.bfloat16
-    _require(qkv.tensor, 'qkv', torch.float32, (qkv.splits, n, (heads + 2 * kv_heads) * head_dim))
+    stored = kv_heads if has_kv else 0
+    if writes and not has_kv:
+        raise ValueError('decode_attention: a step that writes keys and values needs them in qkv')
+    _require(qkv.tensor, 'qkv', torch.float32, (qkv.splits, n, (heads + 2 * stored) * head_dim + extra_columns))
+    if bias is not None:
+        _require(bias, 'bias', torch.float32, ((heads + 2 * stored) * head_dim,))
+    if sinks is not None:
+        _require(sinks, 'sinks', torch.float32, (heads,))
+        unmerged = False
+    coef, every = q_temperature if q_temperature is not None else (0.0, 0)
     _require(block_tables, 'block_tables', torch.int32)
     _require(row_seq, 'row_seq', torch.int32, (n,))
     _require(positions, 'positions', torch.int32, (n,))
@@ -700,8 +711,13 @@ def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps,
                                      block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(workspace), _ptr(out),
                                      n, heads, kv_heads, head_dim, page_size, window_arg, float(scale), part, parts,
                                      DECODE_WAVES, int(n * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= FUSED_PAIRS_MOST_DIM),
-                                     int(bool(rotate_first)), float(softcap or 0.0), _stream()), 'attn_decode_fused')
+                                     int(bool(rotate_first)), float(softcap or 0.0), int(bool(has_kv)), int(extra_columns),
+                                     _ptr(bias), float(coef), int(every), _ptr(sinks), _stream()), 'attn_decode_fused')
     if parts > 1:
+        if sinks is not None:                           # the merge adds the sinks' term
+            _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), n, heads, head_dim, window_arg,
+                                      part, parts, _code(dtype), _ptr(sinks), _stream()), 'attn_merge')
+            return out
         result = Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg, part=part,
                           parts=parts)
         return result if unmerged else result.merge()

@@ -219,7 +219,7 @@ def _declare(lib):
     lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p, p]
     lib.qil_attn_decode_fused_takes.argtypes = [i, i, i, i, i]
     lib.qil_attn_decode_fused_takes.restype = i
-    lib.qil_attn_decode_fused.argtypes = [p, i, p, p, f, p, p, i, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, i, f, p]
+    lib.qil_attn_decode_fused.argtypes = [p, i, p, p, f, p, p, i, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, i, f, i, i, p, f, i, p, p]
     lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
     lib.qil_attn_decode_takes.restype = i
     lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, f, p, p]

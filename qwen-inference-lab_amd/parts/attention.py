@@ -189,6 +189,19 @@ class Attention(Mixer):
         p = self.p
         gate_columns = self.heads * self.padded_dim if self.gate else 0
         stored = self.kv_heads if self.own_kv else 0
+        if ctx.max_query == 1 and self.padded_dim == self.head_dim and \
+                ops.decode_attention_takes(qkv, page_size=cache.page_size, rotation=rotation, dtype=self.dtype, **sizes):
+            # every row alone in its sequence: bias, norm, rotation, temperature and cache write inside the attention kernel
+            attended = ops.decode_attention(
+                qkv, rotation=rotation, positions=ctx.positions, writes=cache.writes, k_cache=cache.k, v_cache=cache.v,
+                page_size=cache.page_size, block_tables=cache.block_tables, row_seq=ctx.row_seq,
+                max_context=ctx.max_context, scale=self.scale, window=self.window, unmerged=False,
+                rotate_first=self.norm_after_rotation, softcap=self.softcap, has_kv=self.own_kv,
+                extra_columns=gate_columns, bias=self.b_qkv_own, q_temperature=self.q_temperature, sinks=p.get('sinks'),
+                **sizes, **norms)
+            if self.gate:
+                attended = ops.sigmoid_gate(attended, qkv, offset=(self.heads + 2 * stored) * self.padded_dim)
+            return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)
         q = ops.qk_norm_rope_store(
             qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,
             k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype, norm_dim=self.head_dim,

@@ -279,3 +279,51 @@ def test_router_with_sigmoid_scores_and_groups_by_their_two_best(dtype, outputs,
     assert torch.equal(chosen.cpu()[clear], want_chosen[clear])
     torch.testing.assert_close(weights.cpu()[clear], want_weights[clear], rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(weights.cpu()[clear].sum(dim=-1), torch.full((int(clear.sum()),), 2.5), rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------ decoding in one kernel
+@pytest.mark.parametrize('lengths,page_size,d,heads,kv_heads,window,rot,splits,extra,biased,temperature,sunk,has_kv', [
+    ([2100, 1, 700, 1290, 64, 2047, 300, 33], 16, 128, 16, 4, None, 0, 8, 16 * 128, True, (0.5, 64), False, True),
+    ([1, 2, 31, 32, 33, 64, 65, 96], 8, 64, 6, 2, 20, 32, 3, 0, False, None, True, True),
+    ([257, 512, 513], 32, 128, 8, 1, 100, 64, 1, 64, True, (1.5, 3), True, True),
+    ([40, 1000, 3000], 16, 64, 16, 1, None, 0, 2, 16 * 64, True, (0.2, 100), False, False),
+])
+def test_decoding_with_queries_made_inside_is_the_two_kernels(lengths, page_size, d, heads, kv_heads, window, rot, splits, extra,
+                                                              biased, temperature, sunk, has_kv):
+    """The decode kernel that makes its queries, new key and new value itself, with what this design adds (the
+    projection's bias, columns of another branch behind q, k and v, the query temperature, sinks, rows of queries
+    only): bit for bit what the q/k kernel followed by the attention kernels leave, results and pages."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(d + heads)
+    rows = len(lengths)
+    stored = kv_heads if has_kv else 0
+    k_cache, v_cache, table, _ = build_cache(lengths, page_size, kv_heads, d, dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    row_seq = torch.arange(rows, dtype=torch.int32).cuda()
+    slots = (table[row_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32)
+    qkv = ops.Partials((torch.randn(splits, rows, (heads + 2 * stored) * d + extra, generator=g) * 0.7).cuda())
+    ones = torch.ones(d).cuda()
+    bias = torch.randn((heads + 2 * stored) * d, generator=g).cuda() if biased else None
+    sinks = torch.linspace(-3.0, 3.0, heads).cuda() if sunk else None
+    rotation = None
+    if rot:
+        from qil_amd.parts import RotaryFrequencies
+        rotation = RotaryFrequencies(rot, 1000.0, device='cuda', scaling=(4.0, 1.0, 4.0, 128)).rotation()
+    sizes = dict(heads=heads, kv_heads=kv_heads, head_dim=d)
+    assert ops.decode_attention_takes(qkv, page_size=page_size, rotation=rotation, dtype=dtype, **sizes)
+    k_two, v_two = k_cache.clone(), v_cache.clone()
+    q = ops.qk_norm_rope_store(qkv, q_weight=ones, k_weight=ones, eps=1e-6, rotation=rotation, positions=positions,
+                               slots=slots if has_kv else None, k_cache=k_two, v_cache=v_two, page_size=page_size, dtype=dtype,
+                               heads=heads, kv_heads=stored, head_dim=d, extra_columns=extra, q_temperature=temperature, bias=bias)
+    want = ops.paged_attention(q, k_cache=k_two, v_cache=v_two, page_size=page_size, block_tables=table, row_seq=row_seq,
+                               positions=positions, cu_seqlens=None, seq_starts=None, single_rows=None, n_seqs=rows,
+                               max_query=1, max_context=max(lengths), scale=d ** -0.5, window=window, sinks=sinks, **sizes)
+    k_one, v_one = k_cache.clone(), v_cache.clone()
+    got = ops.decode_attention(qkv, q_weight=ones, k_weight=ones, eps=1e-6, rotation=rotation, positions=positions,
+                               writes=has_kv, k_cache=k_one, v_cache=v_one, page_size=page_size, block_tables=table,
+                               row_seq=row_seq, max_context=max(lengths), scale=d ** -0.5, window=window, has_kv=has_kv,
+                               extra_columns=extra, bias=bias, q_temperature=temperature, sinks=sinks, **sizes)
+    assert isinstance(got, torch.Tensor) and torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got, want, atol=0, rtol=0)
+    same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))          # NaN-filled pages: compare the bits
+    assert same(k_one, k_two) and same(v_one, v_two), 'the pages differ'
